@@ -343,14 +343,16 @@ class HybridLayer(ctypes.Structure):
                 ("d_decay_channels", c_i32), ("d_a_rank", c_i32), ("d_gate", c_i32), ("d_g_rank", c_i32), ("d_out_scale", c_f32),
                 ("g_width", c_i32), ("mlp_kind", c_i32), ("mlp_ff", c_i32), ("mlp_limit", c_f32), ("mlp_alpha", c_f32),
                 ("a_rot_interleaved", c_i32), ("a_kv_rank", c_i32), ("a_rot_dim", c_i32), ("a_head_gate", c_i32), ("a_conv", c_i32),
-                ("a_norm_whole", c_i32), ("a_v_unit", c_i32), ("a_softcap", c_f32), ("a_talk", c_i32), ("share_with", c_i32)]
+                ("a_norm_whole", c_i32), ("a_v_unit", c_i32), ("a_softcap", c_f32), ("a_talk", c_i32), ("share_with", c_i32),
+                ("a_keep_first", c_i32), ("a_norm_after_rot", c_i32), ("a_head_temp", c_i32), ("in_conv", c_i32),
+                ("moe_experts", c_i32), ("moe_top", c_i32), ("moe_shared_ff", c_i32), ("moe_scale", c_f32)]
 
 
 class HybridConfig(ctypes.Structure):
     """mirror of `mi355_hybrid_config`"""
     _fields_ = [("width", c_i32), ("vocab", c_i32), ("n_layers", c_i32), ("dtype", c_i32), ("block_size", c_i32),
                 ("state_slots", c_i32), ("norm_eps", c_f32), ("unit_eps", c_f32),
-                ("residual_form", c_i32), ("resid_alpha", c_f32), ("norm_groups", c_i32)]
+                ("residual_form", c_i32), ("resid_alpha", c_f32), ("norm_groups", c_i32), ("logit_scale", c_f32)]
 
 
 _sig("mi355_be_state_init", c_i32, [c_vp, c_i32])
@@ -402,6 +404,18 @@ _sig("mi355_hyb_resid_norm", ctypes.c_int, [c_vp, c_vp, c_vp, c_i32, c_vp, c_i32
 _sig("mi355_hyb_gather_group_norm", ctypes.c_int, [c_vp, c_i32, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32, c_f32, c_i64])
 _sig("mi355_hyb_gelu_glu", ctypes.c_int, [c_vp, c_i32, c_vp, c_i32, c_i32, c_i64])
 _sig("mi355_hyb_conv", ctypes.c_int, [c_vp, c_vp, c_i32, c_i32, c_vp, c_vp, c_i64, c_vp, c_vp, c_vp, c_vp] + [c_i32] * 5 + [c_i64])
+_sig("mi355_hyb_pre_norm", ctypes.c_int, [c_vp, c_i32, c_vp, c_vp, c_i32, c_i32, c_f32, c_i64])
+_sig("mi355_hyb_conv_residual", ctypes.c_int, [c_vp, c_i32, c_vp, c_i32, c_i32, c_vp, c_vp, c_i64, c_vp, c_vp, c_vp, c_vp] + [c_i32] * 4 + [c_i64])
+_sig("mi355_hyb_attn_prepare_ex", ctypes.c_int, [c_vp] * 4 + [c_i32] * 4 + [c_vp] * 6 + [c_i32] * 8 + [c_vp, c_f32, c_i32, c_i64])
+_sig("mi355_hyb_masked_attention", ctypes.c_int, [c_vp, c_i32, c_i32, c_i32] + [c_vp] * 8 + [c_i32] * 10 + [c_f32, c_f32, c_i32, c_i32, c_f32,
+                                                                                                      c_i32, c_i32, c_i64])
+_sig("mi355_hyb_moe_route", ctypes.c_int, [c_vp, c_vp, c_vp, c_vp, c_i32, c_vp, c_vp, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_f32, c_f32, c_i64])
+_sig("mi355_hyb_moe_block_rows", c_i32, [c_i32] * 5)
+_sig("mi355_hyb_moe_group", ctypes.c_int, [c_vp, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_i64])
+_sig("mi355_hyb_linear_grouped", ctypes.c_int, [c_vp, c_i32, c_vp, c_i32, c_i32, c_vp, c_vp, c_i64, c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_i64])
+_sig("mi355_hyb_silu_glu", ctypes.c_int, [c_vp, c_i32, c_vp, c_i32, c_i32, c_vp, c_i32, c_i64])
+_sig("mi355_hyb_moe_combine_norm_add", ctypes.c_int, [c_vp] * 8 + [c_i32, c_i32, c_i32, c_f32, c_i64])
+_sig("mi355_hyb_scale_f32", ctypes.c_int, [c_vp, c_f32, c_i64, c_i64])
 
 # the hand-written ctypes mirrors must have the layout the library was built with
 for _id, _cls in ((0, QmmDesc), (1, LlamaConfig), (2, DenseConfig), (3, RopeScaling), (4, HybridConfig), (5, HybridLayer)):

@@ -68,13 +68,27 @@ struct LinArgs {
     int T, N, K;
     int a_vec, w_vec;       // rows may be read 16 bytes at a time
     int64_t a_bs, w_bs, o_bs;   // blockIdx.z = one of several independent products of this shape: element strides of its operands
+    // grouped product (blk != NULL): the rows come in blocks of blk_rows = the kernel's tile height; block b = blockIdx.y multiplies its
+    // rows [b blk_rows, blk[2b + 1]) with matrix blk[2b] (w + blk[2b] w_bs); row r of `a` is read at row_src[r] when row_src != NULL
+    const int32_t* blk; const int32_t* row_src; int blk_rows;
 };
+// the block's matrix and the end of its rows (one past the last); false = nothing to do
+__device__ __forceinline__ bool lin_group(LinArgs& p, int t0, int64_t& w_off) {
+    w_off = (int64_t)blockIdx.z * p.w_bs;
+    if (!p.blk) return true;
+    const int b = t0 / p.blk_rows;
+    const int e = p.blk[2 * b], end = p.blk[2 * b + 1];
+    if (t0 >= end) return false;
+    p.T = end;
+    w_off = (int64_t)e * p.w_bs;
+    return true;
+}
+__device__ __forceinline__ int lin_row(const LinArgs& p, int t) { return p.row_src ? p.row_src[t] : t; }
 template <typename TA> __device__ __forceinline__ void lin_batch(LinArgs& p) {
     const int64_t z = blockIdx.z;
     p.a = static_cast<const TA*>(p.a) + z * p.a_bs;
     p.out += z * p.o_bs;
 }
-template <typename TW> __device__ __forceinline__ const TW* lin_w(const LinArgs& p) { return static_cast<const TW*>(p.w) + (int64_t)blockIdx.z * p.w_bs; }
 
 // Prompt-sized products, bf16 weights.  A workgroup of four waves owns 64 output columns (16 weight rows per wave) and 16 MT tokens;
 // fragments go from global memory / L2 straight into registers: lane (m16, kg) holds operands 8 kg .. 8 kg + 7 of row m16 of a
@@ -84,14 +98,16 @@ template <typename TA, int MT> __global__ __launch_bounds__(256) void linear_bf1
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, m16 = lane & 15, kg = lane >> 4;
     const int n = blockIdx.x * 64 + wave * 16 + m16;
     const int t0 = blockIdx.y * (16 * MT);
-    const uint16_t* wrow = lin_w<uint16_t>(p) + (size_t)(n < p.N ? n : 0) * p.K;
+    int64_t w_off;
+    if (!lin_group(p, t0, w_off)) return;
+    const uint16_t* wrow = static_cast<const uint16_t*>(p.w) + w_off + (size_t)(n < p.N ? n : 0) * p.K;
     const TA* arow[MT];
     bool aok[MT];
 #pragma unroll
     for (int i = 0; i < MT; ++i) {
         const int t = t0 + i * 16 + m16;
         aok[i] = t < p.T;
-        arow[i] = static_cast<const TA*>(p.a) + (size_t)(aok[i] ? t : 0) * p.lda;
+        arow[i] = static_cast<const TA*>(p.a) + (size_t)(aok[i] ? lin_row(p, t) : 0) * p.lda;
     }
     f32x4_t acc[MT];
 #pragma unroll
@@ -128,8 +144,10 @@ __global__ __launch_bounds__(256) void linear_bf16_lds_kernel(LinArgs p) {
     const int wr = wave >> 1, wc = wave & 1;
     const int n0 = blockIdx.x * 128, t0 = blockIdx.y * 128;
     lin_batch<uint16_t>(p);
+    int64_t w_off;
+    if (!lin_group(p, t0, w_off)) return;
     const uint16_t* A = static_cast<const uint16_t*>(p.a);
-    const uint16_t* W = lin_w<uint16_t>(p);
+    const uint16_t* W = static_cast<const uint16_t*>(p.w) + w_off;
     // staging: thread -> rows r0 and r0 + 64 of both slices, 16-byte chunk ch of the 64-byte row
     const int r0 = tid >> 2, ch = tid & 3;
     const uint16_t* asrc[2]; const uint16_t* wsrc[2]; bool aok[2], wok[2];
@@ -137,7 +155,7 @@ __global__ __launch_bounds__(256) void linear_bf16_lds_kernel(LinArgs p) {
     for (int j = 0; j < 2; ++j) {
         const int t = t0 + r0 + 64 * j, n = n0 + r0 + 64 * j;
         aok[j] = t < p.T; wok[j] = n < p.N;
-        asrc[j] = A + (size_t)(aok[j] ? t : 0) * p.lda + ch * 8;
+        asrc[j] = A + (size_t)(aok[j] ? lin_row(p, t) : 0) * p.lda + ch * 8;
         wsrc[j] = W + (size_t)(wok[j] ? n : 0) * p.K + ch * 8;
     }
     uint4 ra[2], rw[2];
@@ -201,9 +219,12 @@ template <typename TA, int NW, int UNR> __global__ __launch_bounds__(64 * NW) vo
     lin_batch<TA>(p);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, m16 = lane & 15, kg = lane >> 4;
     const int n = blockIdx.x * 16 + m16;
-    const bool nok = n < p.N, aok = m16 < p.T;
-    const uint16_t* wrow = lin_w<uint16_t>(p) + (size_t)(nok ? n : 0) * p.K;
-    const TA* arow = static_cast<const TA*>(p.a) + (size_t)(aok ? m16 : 0) * p.lda;
+    const int t0 = blockIdx.y * 16;                                  // a grouped product: block blockIdx.y of 16 rows; else 0
+    int64_t w_off;
+    if (!lin_group(p, t0, w_off)) return;
+    const bool nok = n < p.N, aok = t0 + m16 < p.T;
+    const uint16_t* wrow = static_cast<const uint16_t*>(p.w) + w_off + (size_t)(nok ? n : 0) * p.K;
+    const TA* arow = static_cast<const TA*>(p.a) + (size_t)(aok ? lin_row(p, t0 + m16) : 0) * p.lda;
     f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
     for (int k0 = wave * 32 * UNR; k0 < p.K; k0 += NW * 32 * UNR) {
         uint4 a[UNR], b[UNR];
@@ -226,7 +247,7 @@ template <typename TA, int NW, int UNR> __global__ __launch_bounds__(64 * NW) vo
             float s = 0.f;
 #pragma unroll
             for (int w = 0; w < NW; ++w) s += part[w][v][lane];
-            const int t = 4 * kg + v;
+            const int t = t0 + 4 * kg + v;
             if (nok && t < p.T) p.out[(size_t)t * p.ldo + n] = s + bias;
         }
     }
@@ -239,8 +260,10 @@ __global__ __launch_bounds__(256) void linear_f32_kernel(LinArgs p) {
     const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
     const int n0 = blockIdx.x * 64, t0 = blockIdx.y * 64;
     lin_batch<float>(p);
+    int64_t w_off;
+    if (!lin_group(p, t0, w_off)) return;
     const float* A = static_cast<const float*>(p.a);
-    const float* W = lin_w<float>(p);
+    const float* W = static_cast<const float*>(p.w) + w_off;
     float acc[4][4] = {};
     for (int k0 = 0; k0 < p.K; k0 += 16) {
 #pragma unroll
@@ -248,7 +271,7 @@ __global__ __launch_bounds__(256) void linear_f32_kernel(LinArgs p) {
             const int idx = threadIdx.x + r * 256;            // 1024 elements of each 64 x 16 tile
             const int row = idx >> 4, kk = idx & 15;
             const int k = k0 + kk;
-            As[kk][row] = (t0 + row < p.T && k < p.K) ? A[(size_t)(t0 + row) * p.lda + k] : 0.f;
+            As[kk][row] = (t0 + row < p.T && k < p.K) ? A[(size_t)lin_row(p, t0 + row) * p.lda + k] : 0.f;
             Ws[kk][row] = (n0 + row < p.N && k < p.K) ? W[(size_t)(n0 + row) * p.K + k] : 0.f;
         }
         __syncthreads();
@@ -318,7 +341,7 @@ __global__ __launch_bounds__(256) void norm_add_kernel(float* x, uint16_t* xcopy
 template <typename TO> __global__ __launch_bounds__(256) void gather_norm_kernel(TO* out, const float* x, const int32_t* rows, const float* w, int width, float eps) {
     __shared__ float red[4];
     const int r = blockIdx.x;
-    const float* xr = x + (size_t)rows[r] * width;
+    const float* xr = x + (size_t)(rows ? rows[r] : r) * width;
     float ss = 0.f;
     for (int i = threadIdx.x; i < width; i += blockDim.x) ss += xr[i] * xr[i];
     ss = block_sum(ss, red);
@@ -415,6 +438,9 @@ struct PrepArgs {
     const float* qw; const float* kw; const float* cos_t; const float* sin_t;
     const int64_t* positions; const int64_t* slots;
     int H, G, d, vd, rot; float eps;
+    int interleaved;        // rotated pairs are (2i, 2i + 1) instead of (i, i + rot / 2)
+    int norm_mode;          // 0 none, 1 RMS norm (weights qw / kw or none) before the rotation, 2 weightless RMS norm after it
+    const float* q_scale;   // [H] or NULL: head h's query times q_scale[h]
 };
 // one wave per (token, vector): query heads 0 .. H-1, key heads H .. H+G-1, value heads H+G .. H+2G-1
 template <typename TC> __global__ __launch_bounds__(64) void attn_prepare_kernel(PrepArgs p) {
@@ -435,27 +461,42 @@ template <typename TC> __global__ __launch_bounds__(64) void attn_prepare_kernel
     const float* w = is_q ? p.qw : p.kw;
     float ss = 0.f;
     for (int i = lane; i < p.d; i += 64) { const float v = src[i]; vec[i] = v; ss += v * v; }
-    ss = wave_sum(ss);
-    const float inv = w ? 1.f / sqrtf(ss / (float)p.d + p.eps) : 1.f;
-    __syncthreads();
-    for (int i = lane; i < p.d; i += 64) vec[i] = w ? vec[i] * inv * w[i] : vec[i];
+    if (p.norm_mode == 1 && w) {
+        ss = wave_sum(ss);
+        const float inv = 1.f / sqrtf(ss / (float)p.d + p.eps);
+        __syncthreads();
+        for (int i = lane; i < p.d; i += 64) vec[i] = vec[i] * inv * w[i];
+    }
     __syncthreads();
     TC* dst;
     if (is_q) dst = static_cast<TC*>(p.q_out) + ((size_t)t * p.H + h) * p.d;
     else { if (slot < 0) return; dst = static_cast<TC*>(p.k_pages) + ((size_t)slot * p.G + h) * p.d; }
     const int half = p.rot / 2;
     const int64_t pos = p.positions[t];
+    float* rotated = vec + p.d;
+    float s2 = 0.f;
     for (int i = lane; i < p.d; i += 64) {
         float v = vec[i];
-        if (i < half) {
-            const float c = p.cos_t[pos * half + i], s = p.sin_t[pos * half + i];
-            v = vec[i] * c - vec[i + half] * s;
-        } else if (i < p.rot) {
-            const float c = p.cos_t[pos * half + i - half], s = p.sin_t[pos * half + i - half];
-            v = vec[i] * c + vec[i - half] * s;
+        if (i < p.rot) {
+            if (p.interleaved) {
+                const int pr = i >> 1;
+                const float c = p.cos_t[pos * half + pr], s = p.sin_t[pos * half + pr];
+                v = (i & 1) ? vec[i] * c + vec[i - 1] * s : vec[i] * c - vec[i + 1] * s;
+            } else if (i < half) {
+                const float c = p.cos_t[pos * half + i], s = p.sin_t[pos * half + i];
+                v = vec[i] * c - vec[i + half] * s;
+            } else {
+                const float c = p.cos_t[pos * half + i - half], s = p.sin_t[pos * half + i - half];
+                v = vec[i] * c + vec[i - half] * s;
+            }
         }
-        st<TC>(dst, i, v);
+        rotated[i] = v;
+        s2 += v * v;
     }
+    float mul = 1.f;
+    if (p.norm_mode == 2) mul = 1.f / sqrtf(wave_sum(s2) / (float)p.d + p.eps);
+    if (is_q && p.q_scale) mul *= p.q_scale[h];
+    for (int i = lane; i < p.d; i += 64) st<TC>(dst, i, rotated[i] * mul);
 }
 
 struct AttnArgs {
@@ -467,6 +508,7 @@ struct AttnArgs {
     float softcap;          // > 0: score <- cap tanh(score / cap)
     int cross;              // blockIdx.z = the key/value head whose VALUES this block sums (scores still against the head's own keys)
     int cpk;                // lanes that share a key row when it is read 16 bytes a lane (power of two >= d / elements per 16 bytes)
+    int keep;               // with a window: keys at positions < keep stay visible (the first tokens of the sequence)
 };
 __device__ __forceinline__ float cap_score(float s, float cap) { return cap > 0.f ? cap * tanhf(s / cap) : s; }
 // 16 bytes of a page row as floats (EPV = 8 bf16 or 4 f32)
@@ -507,6 +549,8 @@ template <typename TC, int NW, bool VEC, int DQ, int NV> __global__ __launch_bou
     const int n_new = (int)(p.cu_q[s + 1] - p.cu_q[s]);
     const int pos = (int)p.ctx[s] - n_new + (t - (int)p.cu_q[s]);
     const int lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
+    // the visible keys in one run of indices: the kept first tokens below the window (nkeep of them), then the window [lo, pos]
+    const int nkeep = min(p.keep, lo), n_vis = nkeep + pos - lo + 1;
     const int g = h / (p.H / p.G);
     const int gv0 = p.cross ? (int)blockIdx.z * NV : g, oh0 = p.cross ? h * p.G + gv0 : h;
     const TC* q = static_cast<const TC*>(p.q) + ((size_t)t * p.H + h) * p.d;
@@ -528,9 +572,9 @@ template <typename TC, int NW, bool VEC, int DQ, int NV> __global__ __launch_bou
     for (int n = 0; n < NV; ++n)
 #pragma unroll
         for (int e = 0; e < NACC; ++e) acc[n][e] = 0.f;
-    for (int j0 = lo + wave * 64; j0 <= pos; j0 += NW * 64) {
-        const int j = j0 + lane;
-        const int cnt = min(64, pos - j0 + 1);
+    for (int i0 = wave * 64; i0 < n_vis; i0 += NW * 64) {
+        const int cnt = min(64, n_vis - i0);
+        const int j = lane < cnt ? (i0 + lane < nkeep ? i0 + lane : lo + (i0 + lane - nkeep)) : pos + 1;
         float sc = -INFINITY;
         unsigned page_row = 0;
         if (j <= pos) page_row = bt[j / p.bs] * (unsigned)p.bs + (unsigned)(j % p.bs);
@@ -701,12 +745,15 @@ void window_attention_mfma_kernel(AttnArgs p) {
         for (int c = 0; c < VT; ++c) acc[n][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     const int hi = pos0 + nq - 1;
     const int lo = p.window > 0 ? max(0, pos0 - p.window + 1) : 0;
-    for (int j0 = lo; j0 <= hi; j0 += 64) {
+    // the keys any query of the tile may see, in one run of indices: the kept first tokens below the lowest window, then [lo, hi]
+    const int nkeep = min(p.keep, lo), n_vis = nkeep + hi - lo + 1;
+    auto key_at = [&](int i) { return i < nkeep ? i : (i < n_vis ? lo + (i - nkeep) : hi + 1); };
+    for (int j0 = 0; j0 < n_vis; j0 += 64) {
         // the 64 value rows of this chunk, transposed into LDS (zeros past the end: a stale NaN times a zero weight would poison the sum)
         // (a value head's rows are requested into registers one head ahead of their use: the next head's loads are in flight while the
         // current head multiplies)
         uint4 vreg[VT * 2];
-        const int vkey = j0 + lane;
+        const int vkey = key_at(j0 + lane);
         const bool vkv = vkey <= hi;
         const uint16_t* vrow = V + (vkv ? (size_t)bt[vkey / p.bs] * p.bs + (vkey % p.bs) : 0) * p.v_ld + gv0 * vd;
         auto fetch_values = [&](int n) {
@@ -752,7 +799,7 @@ void window_attention_mfma_kernel(AttnArgs p) {
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt) {
             sacc[kt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-            const int key = j0 + kt * 16 + m16;
+            const int key = key_at(j0 + kt * 16 + m16);
             const bool kv = key <= hi;
             const size_t pr = kv ? (size_t)bt[key / p.bs] * p.bs + (key % p.bs) : 0;
             const uint16_t* kr = K + pr * p.k_ld + g * d + 8 * kg;
@@ -772,8 +819,8 @@ void window_attention_mfma_kernel(AttnArgs p) {
             mx[v] = -INFINITY;
 #pragma unroll
             for (int kt = 0; kt < 4; ++kt) {
-                const int key = j0 + kt * 16 + m16;
-                const bool ok_ = r < nq && key <= qpos && (p.window == 0 || qpos - key < p.window);
+                const int key = key_at(j0 + kt * 16 + m16);
+                const bool ok_ = r < nq && key <= qpos && (p.window == 0 || qpos - key < p.window || key < p.keep);
                 sc[v][kt] = ok_ ? cap_score(sacc[kt][v] * p.scale, p.softcap) : -INFINITY;
                 mx[v] = fmaxf(mx[v], sc[v][kt]);
             }
@@ -854,6 +901,8 @@ struct ConvArgs {
     float* out; const float* proj; int ldp, off; const float* w; float* state; int64_t state_stride;
     const uint32_t* ctx; const uint32_t* cu_q; const int32_t* slots; const int32_t* tok_seq; int C, taps, T;
     int act;                // 0 = none, 1 = silu
+    int add_input;          // the convolution is added to its own input (h + conv(h))
+    uint16_t* out_bf16;     // != NULL: the result goes here as bf16 instead of `out`
 };
 __global__ void conv_silu_kernel(ConvArgs p) {
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -874,7 +923,9 @@ __global__ void conv_silu_kernel(ConvArgs p) {
         }
         acc = fmaf(p.w[(size_t)c * p.taps + i], v, acc);
     }
-    p.out[idx] = p.act ? siluf_(acc) : acc;
+    if (p.add_input) acc += p.proj[(size_t)t * p.ldp + p.off + c];
+    acc = p.act ? siluf_(acc) : acc;
+    if (p.out_bf16) p.out_bf16[idx] = f32_to_bf16(acc); else p.out[idx] = acc;
 }
 // state[j], j = 0 .. taps-2 (oldest first) <- the taps - 1 inputs that end with the portion's last token
 __global__ void conv_state_update_kernel(ConvArgs p, int n_seqs) {
@@ -1265,6 +1316,160 @@ template <typename TO> __global__ void head_gate_kernel(TO* out, const float* in
     st<TO>(out, (size_t)i, gate_in ? in[i] * sigmoidf_(gate_in[(size_t)t * ldg + h]) : in[i]);
 }
 
+
+// ------------------------------------------------------------------------------------------------------------ mixture of experts
+// Routing, one workgroup per token: the normalised row h is built once in LDS (and written out for the experts' products), a wave
+// takes the experts e = wave, wave + 4, ... (f32 router rows . h), then wave 0 makes the softmax, the choice by s + correction
+// (largest first, ties to the lower expert) and the weights s[chosen] * scale.  The shared expert's gate is one more row.
+template <typename TO> __global__ __launch_bounds__(256) void moe_route_kernel(int32_t* ids, float* wts, float* sgate, TO* xn, const float* x,
+                                                                               const float* norm_w, const float* router, const float* corr,
+                                                                               const float* gate_row, int width, int E, int K, float scale,
+                                                                               float eps) {
+    extern __shared__ __align__(16) float rsm[];
+    float* hs = rsm;                       // [width]
+    float* logit = hs + width;             // [E + 1]
+    __shared__ float red[4];
+    const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const float* xr = x + (size_t)t * width;
+    float inv = 1.f;
+    if (norm_w) {
+        float ss = 0.f;
+        for (int i = threadIdx.x; i < width; i += blockDim.x) ss += xr[i] * xr[i];
+        inv = 1.f / sqrtf(block_sum(ss, red) / (float)width + eps);
+    }
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        const float v = norm_w ? xr[i] * inv * norm_w[i] : xr[i];
+        hs[i] = v;
+        if (xn) st<TO>(xn, (size_t)t * width + i, v);
+    }
+    __syncthreads();
+    const int rows = E + (gate_row ? 1 : 0);
+    for (int e = wave; e < rows; e += 4) {
+        const float* g = e < E ? router + (size_t)e * width : gate_row;
+        float acc = 0.f;
+        if ((width & 3) == 0) {
+            for (int i = 4 * lane; i < width; i += 256) {
+                const float4 gv = *reinterpret_cast<const float4*>(g + i), hv = *reinterpret_cast<const float4*>(hs + i);
+                acc = fmaf(hv.x, gv.x, fmaf(hv.y, gv.y, fmaf(hv.z, gv.z, fmaf(hv.w, gv.w, acc))));
+            }
+        } else {
+            for (int i = lane; i < width; i += 64) acc = fmaf(hs[i], g[i], acc);
+        }
+        acc = wave_sum(acc);
+        if (lane == 0) logit[e] = acc;
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    if (gate_row && lane == 0) sgate[t] = sigmoidf_(logit[E]);
+    float m = -INFINITY;
+    for (int e = lane; e < E; e += 64) m = fmaxf(m, logit[e]);
+    m = wave_max(m);
+    float den = 0.f;
+    for (int e = lane; e < E; e += 64) den += expf(logit[e] - m);
+    den = wave_sum(den);
+    // lane owns experts lane, lane + 64, ...: K rounds of (my best untaken choice score) -> wave maximum -> the lowest expert that has it
+    unsigned long long taken = 0ull;                                    // bit i: my expert lane + 64 i is chosen already
+    for (int j = 0; j < K; ++j) {
+        float bv = -INFINITY; int be = 0x7fffffff;
+        for (int e = lane, i = 0; e < E; e += 64, ++i) {
+            const float cv = expf(logit[e] - m) / den + (corr ? corr[e] : 0.f);
+            if (!((taken >> i) & 1ull) && (cv > bv || be == 0x7fffffff)) { bv = cv; be = e; }
+        }
+        const float top = wave_max(bv);
+        int cand = (be != 0x7fffffff && bv == top) ? be : 0x7fffffff;
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) cand = min(cand, __shfl_xor(cand, o));
+        if (lane == (cand & 63)) taken |= 1ull << (cand >> 6);
+        if (lane == 0) {
+            ids[(size_t)t * K + j] = cand;
+            wts[(size_t)t * K + j] = expf(logit[cand] - m) / den * scale;
+        }
+    }
+}
+
+// Grouping on the device, one workgroup: counts per expert, whole blocks of `bm` rows per expert, then every pair takes the next free
+// row of its expert's blocks (rows are independent, so the order inside an expert does not reach any result).
+__global__ __launch_bounds__(1024) void moe_group_kernel(int32_t* pos, int32_t* row_token, int32_t* table, const int32_t* ids, int pairs, int top,
+                                                         int E, int bm, int n_blocks) {
+    extern __shared__ int gsm[];
+    int* cnt = gsm;                 // [E]
+    int* blk0 = cnt + E;            // [E + 1]
+    int* cur = blk0 + E + 1;        // [E]
+    for (int e = threadIdx.x; e < E; e += blockDim.x) { cnt[e] = 0; cur[e] = 0; }
+    __syncthreads();
+    for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
+        int e = ids[p];
+        e = e < 0 ? 0 : (e >= E ? E - 1 : e);
+        atomicAdd(&cnt[e], 1);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        blk0[0] = 0;
+        for (int e = 0; e < E; ++e) blk0[e + 1] = blk0[e] + (cnt[e] + bm - 1) / bm;
+    }
+    __syncthreads();
+    for (int b = threadIdx.x; b < n_blocks; b += blockDim.x) {
+        int lo = 0, hi = E;                                             // the expert e with blk0[e] <= b < blk0[e + 1]
+        if (b >= blk0[E]) { table[2 * b] = 0; table[2 * b + 1] = 0; continue; }
+        while (hi - lo > 1) { const int mid = (lo + hi) >> 1; if (blk0[mid] <= b) lo = mid; else hi = mid; }
+        table[2 * b] = lo;
+        table[2 * b + 1] = bm * blk0[lo] + cnt[lo];
+    }
+    for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
+        int e = ids[p];
+        e = e < 0 ? 0 : (e >= E ? E - 1 : e);
+        const int r = bm * blk0[e] + atomicAdd(&cur[e], 1);
+        pos[p] = r;
+        row_token[r] = p / top;
+    }
+}
+
+template <typename TO> __global__ void silu_glu_kernel(TO* out, const float* gu, int64_t n, int ff, const int32_t* table, int bm) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const int64_t t = i / ff; const int j = (int)(i - t * ff);
+    if (table && t >= table[2 * (t / bm) + 1]) return;                  // a row that no pair landed in
+    st<TO>(out, (size_t)i, siluf_(gu[t * 2 * ff + j]) * gu[t * 2 * ff + ff + j]);
+}
+
+// y[t] = sum_j wts[t, j] rows[pos[t top + j]] + gate[t] shared[t];  x[t] += y / rms(y) * w.  One workgroup per token; y stays in
+// registers between the two passes (width <= 256 x 16).
+__global__ __launch_bounds__(256) void moe_combine_norm_add_kernel(float* x, uint16_t* xcopy, const float* rows, const int32_t* pos,
+                                                                   const float* wts, const float* shared, const float* sgate, const float* w,
+                                                                   int width, int top, float eps) {
+    __shared__ float red[4];
+    const int t = blockIdx.x;
+    float y[16];
+    float ss = 0.f;
+    const float sg = shared ? (sgate ? sgate[t] : 1.f) : 0.f;
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+        const int i = threadIdx.x + 256 * u;
+        float a = 0.f;
+        if (i < width) {
+            for (int j = 0; j < top; ++j) a = fmaf(wts[(size_t)t * top + j], rows[(size_t)pos[(size_t)t * top + j] * width + i], a);
+            if (shared) a = fmaf(sg, shared[(size_t)t * width + i], a);
+        }
+        y[u] = a;
+        ss += a * a;
+    }
+    ss = block_sum(ss, red);
+    const float inv = 1.f / sqrtf(ss / (float)width + eps);
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+        const int i = threadIdx.x + 256 * u;
+        if (i < width) {
+            const float v = x[(size_t)t * width + i] + y[u] * inv * w[i];
+            x[(size_t)t * width + i] = v;
+            if (xcopy) xcopy[(size_t)t * width + i] = f32_to_bf16(v);
+        }
+    }
+}
+__global__ void scale_f32_kernel(float* x, float s, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) x[i] *= s;
+}
+
 int g_attn_mfma = 1;            // mi355_hyb_set_attention_mfma(0): prompt steps take the generic kernel too (A/B, tests of both paths)
 
 #define LAUNCH_OK() do { const hipError_t e_ = hipGetLastError(); if (e_ != hipSuccess) return (int)e_; } while (0)
@@ -1379,15 +1584,27 @@ int mi355_hyb_attn_prepare(void* q_out, void* k_pages, void* v_pages, const floa
                            int32_t v_off, const float* q_norm_w, const float* k_norm_w, const float* cos_t, const float* sin_t,
                            const int64_t* positions, const int64_t* slot_mapping, int32_t T, int32_t heads, int32_t kv_heads,
                            int32_t dim, int32_t vdim, int32_t rot_dims, float eps, int32_t dtype, int64_t stream) {
+    // (the plain form: a norm only where weights are given, before the rotation; rotate-half pairs)
+    return mi355_hyb_attn_prepare_ex(q_out, k_pages, v_pages, proj, ldp, q_off, k_off, v_off, q_norm_w, k_norm_w, cos_t, sin_t, positions,
+                                     slot_mapping, T, heads, kv_heads, dim, vdim, rot_dims, 0, (q_norm_w || k_norm_w) ? 1 : 0, nullptr, eps,
+                                     dtype, stream);
+}
+
+int mi355_hyb_attn_prepare_ex(void* q_out, void* k_pages, void* v_pages, const float* proj, int32_t ldp, int32_t q_off, int32_t k_off,
+                              int32_t v_off, const float* q_norm_w, const float* k_norm_w, const float* cos_t, const float* sin_t,
+                              const int64_t* positions, const int64_t* slot_mapping, int32_t T, int32_t heads, int32_t kv_heads,
+                              int32_t dim, int32_t vdim, int32_t rot_dims, int32_t interleaved, int32_t norm_mode,
+                              const float* q_head_scale, float eps, int32_t dtype, int64_t stream) {
+    if (norm_mode < 0 || norm_mode > 2) return -1;
     if (!q_out || !k_pages || !v_pages || !proj || !positions || !slot_mapping || !is_dt(dtype)) return -1;
     if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || vdim <= 0 || rot_dims < 0 || rot_dims > dim || (rot_dims & 1)) return -1;
     if (rot_dims > 0 && (!cos_t || !sin_t)) return -1;
     if (T <= 0) return 0;
     PrepArgs p{q_out, k_pages, v_pages, proj, ldp, q_off, k_off, v_off, q_norm_w, k_norm_w, cos_t, sin_t, positions, slot_mapping,
-               heads, kv_heads, dim, vdim, rot_dims, eps};
+               heads, kv_heads, dim, vdim, rot_dims, eps, interleaved, norm_mode, q_head_scale};
     const dim3 grid(T, heads + 2 * kv_heads);
-    if (dtype == MI355_DTYPE_F32) attn_prepare_kernel<float><<<grid, 64, dim * sizeof(float), to_stream(stream)>>>(p);
-    else attn_prepare_kernel<uint16_t><<<grid, 64, dim * sizeof(float), to_stream(stream)>>>(p);
+    if (dtype == MI355_DTYPE_F32) attn_prepare_kernel<float><<<grid, 64, 2 * dim * sizeof(float), to_stream(stream)>>>(p);
+    else attn_prepare_kernel<uint16_t><<<grid, 64, 2 * dim * sizeof(float), to_stream(stream)>>>(p);
     LAUNCH_OK(); return 0;
 }
 
@@ -1407,6 +1624,18 @@ int mi355_hyb_window_attention_ex(void* out, int32_t out_dtype, int32_t ldo, int
                                    int32_t T, int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, int32_t block_size,
                                    int32_t max_blocks, int32_t window, float scale, float out_scale, int32_t k_ld, int32_t v_ld,
                                    float softcap, int32_t cross_values, int32_t dtype, int64_t stream) {
+    return mi355_hyb_masked_attention(out, out_dtype, ldo, out_off, q, k_pages, v_pages, block_tables, context_lens, cu_seqlens_q, tok_seq,
+                                      sink, num_seqs, T, heads, kv_heads, dim, vdim, block_size, max_blocks, window, 0, scale, out_scale,
+                                      k_ld, v_ld, softcap, cross_values, dtype, stream);
+}
+
+int mi355_hyb_masked_attention(void* out, int32_t out_dtype, int32_t ldo, int32_t out_off, const void* q, const void* k_pages,
+                               const void* v_pages, const uint32_t* block_tables, const uint32_t* context_lens,
+                               const uint32_t* cu_seqlens_q, const int32_t* tok_seq, const float* sink, int32_t num_seqs,
+                               int32_t T, int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, int32_t block_size,
+                               int32_t max_blocks, int32_t window, int32_t keep_first, float scale, float out_scale, int32_t k_ld,
+                               int32_t v_ld, float softcap, int32_t cross_values, int32_t dtype, int64_t stream) {
+    if (keep_first < 0) return -1;
     if (!out || !q || !k_pages || !v_pages || !block_tables || !context_lens || !cu_seqlens_q || !tok_seq) return -1;
     if (!is_dt(dtype) || !is_dt(out_dtype) || heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || vdim <= 0) return -1;
     if (block_size <= 0 || max_blocks <= 0 || window < 0 || softcap < 0.f) return -1;
@@ -1424,6 +1653,7 @@ int mi355_hyb_window_attention_ex(void* out, int32_t out_dtype, int32_t ldo, int
     const bool vec = dim % epv == 0 && vdim % epv == 0 && vdim / epv <= 64 && dim / epv <= 64 && (uintptr_t)k_pages % 16 == 0 && (uintptr_t)v_pages % 16 == 0 &&
                      k_ld % epv == 0 && v_ld % epv == 0;
     p.cpk = 64;
+    p.keep = window > 0 ? keep_first : 0;
     if (vec) { int c = 1; while (c < vdim / epv) c <<= 1; p.cp2 = c; c = 1; while (c < dim / epv) c <<= 1; p.cpk = c; }
     else if (vdim > 512) return -1;
     // prompt-sized steps over bf16 pages: the matrix-core kernel (a tile of 16 tokens never spans two sequences)
@@ -1490,7 +1720,21 @@ int mi355_hyb_conv(float* out, const float* proj, int32_t ldp, int32_t off, cons
     if (!out || !proj || !w || !conv_state || !context_lens || !cu_seqlens_q || !state_slots || !tok_seq) return -1;
     if (channels <= 0 || taps < 1 || taps > 16) return -1;
     if (T <= 0) return 0;
-    ConvArgs p{out, proj, ldp, off, w, const_cast<float*>(conv_state), state_stride, context_lens, cu_seqlens_q, state_slots, tok_seq, channels, taps, T, act};
+    ConvArgs p{out, proj, ldp, off, w, const_cast<float*>(conv_state), state_stride, context_lens, cu_seqlens_q, state_slots, tok_seq, channels, taps, T, act, 0, nullptr};
+    const int64_t n = (int64_t)T * channels;
+    conv_silu_kernel<<<(unsigned)((n + 255) / 256), 256, 0, to_stream(stream)>>>(p);
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_conv_residual(void* out, int32_t out_dtype, const float* in, int32_t ld, int32_t off, const float* w, const float* conv_state,
+                            int64_t state_stride, const uint32_t* context_lens, const uint32_t* cu_seqlens_q, const int32_t* state_slots,
+                            const int32_t* tok_seq, int32_t num_seqs, int32_t T, int32_t channels, int32_t taps, int64_t stream) {
+    if (!out || !in || !w || !conv_state || !context_lens || !cu_seqlens_q || !state_slots || !tok_seq || !is_dt(out_dtype)) return -1;
+    if (channels <= 0 || taps < 1 || taps > 16 || ld < off + channels) return -1;
+    if (T <= 0) return 0;
+    const bool f = out_dtype == MI355_DTYPE_F32;
+    ConvArgs p{f ? (float*)out : nullptr, in, ld, off, w, const_cast<float*>(conv_state), state_stride, context_lens, cu_seqlens_q, state_slots,
+               tok_seq, channels, taps, T, 0, 1, f ? nullptr : (uint16_t*)out};
     const int64_t n = (int64_t)T * channels;
     conv_silu_kernel<<<(unsigned)((n + 255) / 256), 256, 0, to_stream(stream)>>>(p);
     LAUNCH_OK(); return 0;
@@ -1501,7 +1745,7 @@ int mi355_hyb_conv_state_update(float* conv_state, int64_t state_stride, const f
                                 int32_t num_seqs, int32_t channels, int32_t taps, int64_t stream) {
     if (!conv_state || !proj || !context_lens || !cu_seqlens_q || !state_slots || channels <= 0 || taps < 1 || taps > 16) return -1;
     if (num_seqs <= 0 || taps == 1) return 0;
-    ConvArgs p{nullptr, proj, ldp, off, nullptr, conv_state, state_stride, context_lens, cu_seqlens_q, state_slots, nullptr, channels, taps, 0, 0};
+    ConvArgs p{nullptr, proj, ldp, off, nullptr, conv_state, state_stride, context_lens, cu_seqlens_q, state_slots, nullptr, channels, taps, 0, 0, 0, nullptr};
     const int n = num_seqs * channels;
     conv_state_update_kernel<<<(n + 255) / 256, 256, 0, to_stream(stream)>>>(p, num_seqs);
     LAUNCH_OK(); return 0;
@@ -1644,6 +1888,109 @@ int mi355_hyb_head_gate(void* out, int32_t out_dtype, const float* in, const flo
     const unsigned grid = (unsigned)((n + 255) / 256);
     if (out_dtype == MI355_DTYPE_F32) head_gate_kernel<float><<<grid, 256, 0, to_stream(stream)>>>((float*)out, in, gate_in, ldg, n, heads, vdim);
     else head_gate_kernel<uint16_t><<<grid, 256, 0, to_stream(stream)>>>((uint16_t*)out, in, gate_in, ldg, n, heads, vdim);
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_pre_norm(void* out, int32_t out_dtype, const float* x, const float* w, int32_t T, int32_t width, float eps, int64_t stream) {
+    if (!out || !x || !w || !is_dt(out_dtype) || width <= 0) return -1;
+    if (T <= 0) return 0;
+    if (out_dtype == MI355_DTYPE_F32) gather_norm_kernel<float><<<T, 256, 0, to_stream(stream)>>>((float*)out, x, nullptr, w, width, eps);
+    else gather_norm_kernel<uint16_t><<<T, 256, 0, to_stream(stream)>>>((uint16_t*)out, x, nullptr, w, width, eps);
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_scale_f32(float* x, float s, int64_t n, int64_t stream) {
+    if (!x) return -1;
+    if (n <= 0) return 0;
+    scale_f32_kernel<<<(unsigned)((n + 255) / 256), 256, 0, to_stream(stream)>>>(x, s, n);
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_moe_route(int32_t* expert_ids, float* weights, float* shared_gate, void* xn, int32_t out_dtype, const float* x,
+                        const float* norm_w, const float* router, const float* correction, const float* gate_row, int32_t T,
+                        int32_t width, int32_t experts, int32_t top, float scale, float eps, int64_t stream) {
+    if (!expert_ids || !weights || !x || !router || width <= 0 || experts < 1 || experts > 4096 || top < 1 || top > experts) return -1;
+    if ((gate_row && !shared_gate) || (xn && !is_dt(out_dtype))) return -1;
+    if (T <= 0) return 0;
+    const size_t lds = (size_t)(width + experts + 1) * sizeof(float);
+    if (lds > 60000) return -1;
+    if (xn && out_dtype == MI355_DTYPE_BF16)
+        moe_route_kernel<uint16_t><<<T, 256, lds, to_stream(stream)>>>(expert_ids, weights, shared_gate, (uint16_t*)xn, x, norm_w, router, correction,
+                                                                      gate_row, width, experts, top, scale, eps);
+    else
+        moe_route_kernel<float><<<T, 256, lds, to_stream(stream)>>>(expert_ids, weights, shared_gate, (float*)xn, x, norm_w, router, correction,
+                                                                   gate_row, width, experts, top, scale, eps);
+    LAUNCH_OK(); return 0;
+}
+
+int32_t mi355_hyb_moe_block_rows(int32_t pairs, int32_t experts, int32_t n, int32_t k, int32_t dtype) {
+    if (dtype == MI355_DTYPE_F32) return 64;                            // the f32 product's tile
+    if (experts < 1) experts = 1;
+    const int avg = pairs / experts;
+    if (avg <= 16) return 16;
+    if (avg <= 96 || k % 32 != 0) return 64;
+    return 128;
+}
+
+int mi355_hyb_moe_group(int32_t* pos, int32_t* row_token, int32_t* block_table, const int32_t* expert_ids, int32_t pairs, int32_t top,
+                        int32_t experts, int32_t block_rows, int32_t n_blocks, int64_t stream) {
+    if (pairs <= 0) return 0;
+    if (!pos || !row_token || !block_table || !expert_ids || top < 1 || experts < 1 || experts > 4096 || block_rows < 1) return -1;
+    if (n_blocks < (pairs + block_rows - 1) / block_rows + experts) return -1;
+    moe_group_kernel<<<1, 1024, (size_t)(3 * experts + 1) * sizeof(int), to_stream(stream)>>>(pos, row_token, block_table, expert_ids, pairs, top,
+                                                                                              experts, block_rows, n_blocks);
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_linear_grouped(float* out, int32_t ldo, const void* a, int32_t a_dtype, int32_t lda, const int32_t* row_token, const void* w,
+                             int64_t w_bs, const int32_t* block_table, int32_t block_rows, int32_t n_blocks, int32_t n, int32_t k,
+                             int32_t dtype, int64_t stream) {
+    if (!out || !a || !w || !block_table || n <= 0 || k <= 0 || ldo < n || lda < k || w_bs < 0 || !is_dt(dtype) || !is_dt(a_dtype)) return -1;
+    if (n_blocks <= 0) return 0;
+    if (n_blocks > 65535) return -1;
+    LinArgs p{out, ldo, a, lda, w, nullptr, n_blocks * block_rows, n, k, 0, 0, 0, w_bs, 0, block_table, row_token, block_rows};
+    hipStream_t st_ = to_stream(stream);
+    if (dtype == MI355_DTYPE_F32) {
+        if (a_dtype != MI355_DTYPE_F32 || block_rows != 64) return -1;
+        linear_f32_kernel<<<dim3((n + 63) / 64, n_blocks, 1), 256, 0, st_>>>(p);
+        LAUNCH_OK(); return 0;
+    }
+    const int a_bytes = a_dtype == MI355_DTYPE_F32 ? 4 : 2;
+    p.w_vec = (k % 8 == 0) && ((uintptr_t)w % 16 == 0) && (w_bs % 8 == 0);
+    p.a_vec = ((size_t)lda * a_bytes % 16 == 0) && ((uintptr_t)a % 16 == 0);
+    const bool af = a_dtype == MI355_DTYPE_F32;
+    if (block_rows == 16) {
+        const dim3 grid((n + 15) / 16, n_blocks, 1);
+        if (k >= 2048) { if (af) linear_bf16_stream_kernel<float, 4, 4><<<grid, 256, 0, st_>>>(p); else linear_bf16_stream_kernel<uint16_t, 4, 4><<<grid, 256, 0, st_>>>(p); }
+        else { if (af) linear_bf16_stream_kernel<float, 2, 2><<<grid, 128, 0, st_>>>(p); else linear_bf16_stream_kernel<uint16_t, 2, 2><<<grid, 128, 0, st_>>>(p); }
+    } else if (block_rows == 64) {
+        const dim3 grid((n + 63) / 64, n_blocks, 1);
+        if (af) linear_bf16_tile_kernel<float, 4><<<grid, 256, 0, st_>>>(p); else linear_bf16_tile_kernel<uint16_t, 4><<<grid, 256, 0, st_>>>(p);
+    } else if (block_rows == 128 && !af && p.a_vec && p.w_vec && k % 32 == 0) {
+        linear_bf16_lds_kernel<<<dim3((n + 127) / 128, n_blocks, 1), 256, 0, st_>>>(p);
+    } else {
+        return -1;
+    }
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_silu_glu(void* out, int32_t out_dtype, const float* gu, int32_t rows, int32_t ff, const int32_t* block_table,
+                       int32_t block_rows, int64_t stream) {
+    if (!out || !gu || ff <= 0 || !is_dt(out_dtype) || (block_table && block_rows < 1)) return -1;
+    const int64_t n = (int64_t)rows * ff;
+    if (n <= 0) return 0;
+    const unsigned grid = (unsigned)((n + 255) / 256);
+    if (out_dtype == MI355_DTYPE_F32) silu_glu_kernel<float><<<grid, 256, 0, to_stream(stream)>>>((float*)out, gu, n, ff, block_table, block_rows);
+    else silu_glu_kernel<uint16_t><<<grid, 256, 0, to_stream(stream)>>>((uint16_t*)out, gu, n, ff, block_table, block_rows);
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_moe_combine_norm_add(float* x, void* xcopy, const float* y_rows, const int32_t* pos, const float* weights,
+                                   const float* y_shared, const float* shared_gate, const float* w, int32_t T, int32_t width, int32_t top,
+                                   float eps, int64_t stream) {
+    if (!x || !y_rows || !pos || !weights || !w || width <= 0 || width > 4096 || top < 1) return -1;
+    if (T <= 0) return 0;
+    moe_combine_norm_add_kernel<<<T, 256, 0, to_stream(stream)>>>(x, (uint16_t*)xcopy, y_rows, pos, weights, y_shared, shared_gate, w, width, top, eps);
     LAUNCH_OK(); return 0;
 }
 

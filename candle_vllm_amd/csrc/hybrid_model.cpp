@@ -2,7 +2,9 @@
 // (sliding-window attention with a sink, gated delta rule, minGRU, attention and delta rule side by side, latent attention, or
 // attention behind a short convolution with mixed head weights) and an optional feed-forward; x <- x + norm(mixer(x)),
 // x <- x + norm(ff(x)) -- or, with residual_form 1, x <- norm(alpha x + mixer(x)), x <- norm(alpha x + ff(x)) -- the sublayers read
-// x itself.  A layer may run on another layer's weights (share_with) and still owns its pages and state.  Like the llama-family host layers
+// x itself; residual_form 2 puts a norm on both sides, x <- x + norm(sub(pre_norm(x))), optionally with a short causal convolution
+// added to the mixer's input.  The feed-forward is a dense gate/up form or a mixture of experts (router, grouped expert products over
+// device-built blocks, shared expert).  A layer may run on another layer's weights (share_with) and still owns its pages and state.  Like the llama-family host layers
 // (host_model.cpp, dense_model.cpp) it owns the weights, the K/V pages and the activation buffers and enqueues one step on a
 // stream; unlike them it owns a pool of recurrent state (one slot per live sequence, handed out by the block engine) and runs
 // prompts, portions of prompts and decoded tokens through the same launches.
@@ -28,6 +30,7 @@ int mi355_hyb_fill_f32(float*, float, int64_t, int64_t);
 int mi355_hyb_embed(float*, void*, const void*, const uint32_t*, int32_t, int32_t, int32_t, int32_t, int64_t);
 int mi355_hyb_gather_norm(void*, int32_t, const float*, const int32_t*, const float*, int32_t, int32_t, float, int64_t);
 }
+#define MOE_MAX_BLOCK_ROWS 128
 
 namespace {
 
@@ -46,6 +49,7 @@ struct HLayer {
     float *cos_t = nullptr, *sin_t = nullptr; int n_pos = 0;
     void *k_pages = nullptr, *v_pages = nullptr;
     int64_t conv_off = 0, state_off = 0;          // floats from the start of a slot
+    int64_t in_conv_off = 0;                      // the input convolution's last rows
     bool has_attn() const { return c.mixer == MI355_HYB_MIX_PARALLEL || c.mixer == MI355_HYB_MIX_ATTENTION; }
     bool has_delta() const { return c.mixer == MI355_HYB_MIX_PARALLEL || c.mixer == MI355_HYB_MIX_DELTA; }
     bool is_latent() const { return c.mixer == MI355_HYB_MIX_LATENT; }
@@ -71,6 +75,12 @@ struct HModel {
     float *prep = nullptr, *x = nullptr, *proj = nullptr, *aux1 = nullptr, *aux2 = nullptr, *conv = nullptr, *o = nullptr, *y = nullptr, *gu = nullptr;
     void *xcopy = nullptr, *q = nullptr, *mix = nullptr, *act = nullptr, *xn = nullptr, *att = nullptr;
     int32_t* tok_seq = nullptr;
+    // residual form 2 / input convolution: what the sublayer's first product reads; mixture of experts: routing and the gathered rows
+    void *pre = nullptr, *moe_act = nullptr;
+    float *moe_gu = nullptr, *moe_y = nullptr, *moe_wts = nullptr, *moe_sgate = nullptr;
+    int32_t *moe_ids = nullptr, *moe_pos = nullptr, *moe_row_token = nullptr, *moe_table = nullptr;
+    bool need_pre = false;
+    int max_moe_top = 0, max_moe_experts = 0, max_moe_ff = 0;
     int max_in_rows = 0, max_aux1 = 0, max_aux2 = 0, max_conv = 0, max_o = 0, max_q = 0, max_mix = 0, max_ff = 0, max_prep = 0, max_att = 0;
     // captured steps (mi355_hybrid_forward_graph): one hipGraph per (device input pointers, counts); whatever re-allocates a buffer a
     // step touches drops them all
@@ -143,7 +153,10 @@ bool layer_ok(const mi355_hybrid_layer& c) {
         if (c.d_gate != MI355_HYB_GATE_SIGMOID_LR && c.d_gate != MI355_HYB_GATE_SILU) return false;
     }
     if (c.mixer == MI355_HYB_MIX_MINGRU && c.g_width <= 0) return false;
-    if (c.mlp_kind < 0 || c.mlp_kind > 2 || (c.mlp_kind && c.mlp_ff <= 0)) return false;
+    if (c.mlp_kind < 0 || c.mlp_kind > 3 || (c.mlp_kind && c.mlp_ff <= 0)) return false;
+    if (c.mlp_kind == 3 && (c.moe_experts < 1 || c.moe_experts > 4096 || c.moe_top < 1 || c.moe_top > c.moe_experts || c.moe_shared_ff < 0)) return false;
+    if (c.a_keep_first < 0 || c.in_conv < 0 || c.in_conv > 16) return false;
+    if ((c.a_keep_first || c.a_norm_after_rot || c.a_head_temp) && !attn) return false;      // switches of the plain attention branch
     return true;
 }
 
@@ -151,7 +164,8 @@ bool layer_ok(const mi355_hybrid_layer& c) {
 bool is_matrix(int which) {
     switch (which) {
         case MI355_HW_EMBED: case MI355_HW_HEAD: case MI355_HW_IN_PROJ: case MI355_HW_OUT_PROJ: case MI355_HW_D_A2: case MI355_HW_D_G2:
-        case MI355_HW_MLP_GATE_UP: case MI355_HW_MLP_DOWN: case MI355_HW_L_UKT: case MI355_HW_L_UV: return true;
+        case MI355_HW_MLP_GATE_UP: case MI355_HW_MLP_DOWN: case MI355_HW_L_UKT: case MI355_HW_L_UV:
+        case MI355_HW_MOE_GATE_UP: case MI355_HW_MOE_DOWN: return true;
         default: return false;
     }
 }
@@ -173,9 +187,17 @@ int64_t expected_elems(const HModel* m, int layer, int which) {
         case MI355_HW_IN_BIAS: return L.in_rows;
         case MI355_HW_OUT_PROJ: return (int64_t)W * L.out_k;
         case MI355_HW_A_QNORM: if (L.is_conv_attn()) return c.a_qk_norm ? c.a_heads * c.a_dim : -1;
-                               return L.has_attn() && c.a_qk_norm ? c.a_dim : -1;
+                               return L.has_attn() && c.a_qk_norm && !c.a_norm_after_rot ? c.a_dim : -1;
         case MI355_HW_A_KNORM: if (L.is_conv_attn()) return c.a_qk_norm ? c.a_kv_heads * c.a_dim : -1;
-                               return L.has_attn() && c.a_qk_norm ? c.a_dim : -1;
+                               return L.has_attn() && c.a_qk_norm && !c.a_norm_after_rot ? c.a_dim : -1;
+        case MI355_HW_A_TEMP: return L.has_attn() && c.a_head_temp ? c.a_heads : -1;
+        case MI355_HW_PRE_NORM1: return m->cfg.residual_form == 2 ? W : -1;
+        case MI355_HW_PRE_NORM2: return m->cfg.residual_form == 2 && c.mlp_kind ? W : -1;
+        case MI355_HW_IN_CONV: return c.in_conv ? (int64_t)W * c.in_conv : -1;
+        case MI355_HW_MOE_ROUTER: return c.mlp_kind == 3 ? (int64_t)(c.moe_experts + (c.moe_shared_ff ? 1 : 0)) * W : -1;
+        case MI355_HW_MOE_CORRECTION: return c.mlp_kind == 3 ? c.moe_experts : -1;
+        case MI355_HW_MOE_GATE_UP: return c.mlp_kind == 3 ? (int64_t)c.moe_experts * 2 * c.mlp_ff * W : -1;
+        case MI355_HW_MOE_DOWN: return c.mlp_kind == 3 ? (int64_t)c.moe_experts * W * c.mlp_ff : -1;
         case MI355_HW_A_SINK: return (L.has_attn() || L.is_latent()) && c.a_has_sink ? c.a_heads : -1;
         case MI355_HW_A_CONV: return L.is_conv_attn() ? (int64_t)L.a_conv_channels() * c.a_conv : -1;
         case MI355_HW_A_TALK: return L.is_conv_attn() && c.a_talk ? c.a_heads * c.a_heads : -1;
@@ -188,8 +210,10 @@ int64_t expected_elems(const HModel* m, int layer, int which) {
         case MI355_HW_D_NORM: return L.has_delta() ? c.d_vdim : -1;
         case MI355_HW_D_A2: return L.has_delta() && c.d_decay_channels ? (int64_t)c.d_heads * c.d_dim * c.d_a_rank : -1;
         case MI355_HW_D_G2: return L.has_delta() && c.d_gate == MI355_HYB_GATE_SIGMOID_LR ? (int64_t)c.d_heads * c.d_vdim * c.d_g_rank : -1;
-        case MI355_HW_MLP_GATE_UP: return c.mlp_kind ? (int64_t)2 * c.mlp_ff * W : -1;
-        case MI355_HW_MLP_DOWN: return c.mlp_kind ? (int64_t)W * c.mlp_ff : -1;
+        case MI355_HW_MLP_GATE_UP: if (c.mlp_kind == 3) return c.moe_shared_ff ? (int64_t)2 * c.moe_shared_ff * W : -1;
+                                   return c.mlp_kind ? (int64_t)2 * c.mlp_ff * W : -1;
+        case MI355_HW_MLP_DOWN: if (c.mlp_kind == 3) return c.moe_shared_ff ? (int64_t)W * c.moe_shared_ff : -1;
+                                return c.mlp_kind ? (int64_t)W * c.mlp_ff : -1;
         default: return -1;
     }
 }
@@ -244,6 +268,19 @@ int ensure_capacity(HModel* m, int T, int n_out) {
         HCHECK(grow(m->act, t * (size_t)m->max_ff * m->esize()));
         HCHECK(grow(m->att, t * (size_t)m->max_att * m->esize()));
         HCHECK(grow(m->tok_seq, t * 4));
+        if (m->need_pre) HCHECK(grow(m->pre, t * W * m->esize()));
+        if (m->max_moe_experts) {
+            const size_t pairs = t * m->max_moe_top, rows = pairs + (size_t)(m->max_moe_experts + 1) * MOE_MAX_BLOCK_ROWS;
+            HCHECK(grow(m->moe_ids, pairs * 4));
+            HCHECK(grow(m->moe_pos, pairs * 4));
+            HCHECK(grow(m->moe_wts, pairs * 4));
+            HCHECK(grow(m->moe_sgate, t * 4));
+            HCHECK(grow(m->moe_row_token, rows * 4));
+            HCHECK(grow(m->moe_table, (pairs / 16 + m->max_moe_experts + 2) * 2 * 4));
+            HCHECK(grow(m->moe_gu, rows * 2 * m->max_moe_ff * 4));
+            HCHECK(grow(m->moe_act, rows * m->max_moe_ff * m->esize()));
+            HCHECK(grow(m->moe_y, rows * W * 4));
+        }
         m->cap_t = T;
     }
     if (n_out > m->cap_out) {
@@ -280,9 +317,12 @@ void* mi355_hybrid_create(const mi355_hybrid_config* cfg, const mi355_hybrid_lay
             if (std::memcmp(&a, &b, sizeof(a)) != 0) return nullptr;
         }
     }
-    if (cfg->residual_form < 0 || cfg->residual_form > 1 || cfg->norm_groups < 0 || (cfg->norm_groups > 1 && cfg->width % cfg->norm_groups)) return nullptr;
+    if (cfg->residual_form < 0 || cfg->residual_form > 2 || cfg->norm_groups < 0 || (cfg->norm_groups > 1 && cfg->width % cfg->norm_groups)) return nullptr;
+    for (int i = 0; i < cfg->n_layers; ++i)                        // the experts' outputs are combined in front of an output norm
+        if (layers[i].mlp_kind == 3 && (cfg->residual_form == 1 || cfg->width > 4096)) return nullptr;
     HModel* m = new HModel();
     m->cfg = *cfg;
+    m->need_pre = cfg->residual_form == 2;
     m->layers.resize(cfg->n_layers);
     int64_t off = 0;
     for (int i = 0; i < cfg->n_layers; ++i) {
@@ -318,7 +358,13 @@ void* mi355_hybrid_create(const mi355_hybrid_config* cfg, const mi355_hybrid_lay
             L.state_off = off; off += (int64_t)c.d_heads * c.d_dim * c.d_vdim;
         }
         if (c.mixer == MI355_HYB_MIX_MINGRU) { L.state_off = off; off += c.g_width; }
-        if (c.mlp_kind) m->max_ff = std::max(m->max_ff, c.mlp_ff);
+        if (c.in_conv) { L.in_conv_off = off; off += (int64_t)cfg->width * (c.in_conv - 1); m->need_pre = true; }
+        if (c.mlp_kind == 3) {
+            m->max_moe_experts = std::max(m->max_moe_experts, c.moe_experts);
+            m->max_moe_top = std::max(m->max_moe_top, c.moe_top);
+            m->max_moe_ff = std::max(m->max_moe_ff, c.mlp_ff);
+            m->max_ff = std::max(m->max_ff, c.moe_shared_ff);
+        } else if (c.mlp_kind) m->max_ff = std::max(m->max_ff, c.mlp_ff);
     }
     m->slot_floats = std::max<int64_t>(off, 1);
     return m;
@@ -334,7 +380,9 @@ void mi355_hybrid_destroy(void* mp) {
         for (void* p : {(void*)L.cos_t, (void*)L.sin_t, L.k_pages, L.v_pages}) if (p) (void)hipFree(p);
     }
     for (void* p : {m->embed.p, m->final_norm.p, m->head.p, (void*)m->state, (void*)m->prep, (void*)m->x, (void*)m->proj, (void*)m->aux1, (void*)m->aux2,
-                    (void*)m->conv, (void*)m->o, (void*)m->y, (void*)m->gu, m->xcopy, m->q, m->mix, m->act, m->xn, m->att, (void*)m->tok_seq})
+                    (void*)m->conv, (void*)m->o, (void*)m->y, (void*)m->gu, m->xcopy, m->q, m->mix, m->act, m->xn, m->att, (void*)m->tok_seq,
+                    m->pre, m->moe_act, (void*)m->moe_gu, (void*)m->moe_y, (void*)m->moe_wts, (void*)m->moe_sgate, (void*)m->moe_ids,
+                    (void*)m->moe_pos, (void*)m->moe_row_token, (void*)m->moe_table})
         if (p) (void)hipFree(p);
     delete m;
 }
@@ -423,7 +471,7 @@ static int forward_check(HModel* m, const uint32_t* tokens, const int64_t* posit
             const int need[] = {MI355_HW_NORM1, MI355_HW_IN_PROJ, MI355_HW_OUT_PROJ};
             for (int s : need) if (!L.w[s].p) return -3;
             for (int s = MI355_HW_NORM2; s < MI355_HW_COUNT; ++s)
-                if (s != MI355_HW_IN_BIAS && expected_elems(m, (int)(&L - m->layers.data()), s) > 0 && !L.w[s].p) return -3;
+                if (s != MI355_HW_IN_BIAS && s != MI355_HW_MOE_CORRECTION && expected_elems(m, (int)(&L - m->layers.data()), s) > 0 && !L.w[s].p) return -3;
         }
         if (L.uses_pages() && (!L.k_pages || (L.rotates() && WL.n_pos < max_context_len))) return -4;
     }
@@ -437,27 +485,44 @@ static int forward_enqueue(HModel* m, const uint32_t* tokens, const int64_t* pos
     const int W = m->cfg.width, dt = m->cfg.dtype;
     const float eps = m->cfg.norm_eps;
     const bool bf = m->bf16();
-    void* xin = bf ? m->xcopy : (void*)m->x;                       // what the sublayers' first product reads
+    const bool sandwich = m->cfg.residual_form == 2;                // a norm in front of every sublayer: nothing reads a copy of x
+    void* xcopy = (bf && !sandwich) ? m->xcopy : nullptr;
+    void* xin = sandwich ? m->pre : (bf ? m->xcopy : (void*)m->x);  // what the sublayers' first product reads
     const int xin_dt = bf ? MI355_DTYPE_BF16 : MI355_DTYPE_F32;
     HCHECK(mi355_hyb_token_seq(m->tok_seq, cu_seqlens_q, num_seqs, stream));
-    HCHECK(mi355_hyb_embed(m->x, bf ? m->xcopy : nullptr, m->embed.p, tokens, T, W, m->cfg.vocab, dt, stream));
+    HCHECK(mi355_hyb_embed(m->x, xcopy, m->embed.p, tokens, T, W, m->cfg.vocab, dt, stream));
     for (size_t li = 0; li < m->layers.size(); ++li) {
         HLayer& L = m->layers[li];
         const mi355_hybrid_layer& c = L.c;
         const HLayer& WL = c.share_with ? m->layers[c.share_with - 1] : L;          // whose weights (and rope tables) the layer runs on
         auto f = [&](int which) { return static_cast<const float*>(WL.w[which].p); };
         const int ldp = L.in_rows;
-        HCHECK(mi355_hyb_linear(m->proj, ldp, xin, xin_dt, W, WL.w[MI355_HW_IN_PROJ].p, f(MI355_HW_IN_BIAS), T, L.in_rows, W, dt, stream));
+        const void* min_ = xin;                                         // the mixer's input
+        if (c.in_conv) {
+            // h + conv(h): h = the normed x (form 2; f32 in m->y, free until the output projection) or x itself
+            const float* h = m->x;
+            if (sandwich) { HCHECK(mi355_hyb_pre_norm(m->y, MI355_DTYPE_F32, m->x, f(MI355_HW_PRE_NORM1), T, W, eps, stream)); h = m->y; }
+            float* cst = m->state + L.in_conv_off;
+            HCHECK(mi355_hyb_conv_residual(m->pre, dt, h, W, 0, f(MI355_HW_IN_CONV), cst, m->slot_floats, context_lens, cu_seqlens_q, state_slots,
+                                           m->tok_seq, num_seqs, T, W, c.in_conv, stream));
+            HCHECK(mi355_hyb_conv_state_update(cst, m->slot_floats, h, W, 0, context_lens, cu_seqlens_q, state_slots, num_seqs, W, c.in_conv, stream));
+            min_ = m->pre;
+        } else if (sandwich) {
+            HCHECK(mi355_hyb_pre_norm(m->pre, dt, m->x, f(MI355_HW_PRE_NORM1), T, W, eps, stream));
+        }
+        HCHECK(mi355_hyb_linear(m->proj, ldp, min_, xin_dt, W, WL.w[MI355_HW_IN_PROJ].p, f(MI355_HW_IN_BIAS), T, L.in_rows, W, dt, stream));
         int mix_col = 0;
         if (L.has_attn()) {
-            HCHECK(mi355_hyb_attn_prepare(m->q, L.k_pages, L.v_pages, m->proj, ldp, L.off[P_AQ], L.off[P_AK], L.off[P_AV],
-                                          c.a_qk_norm ? f(MI355_HW_A_QNORM) : nullptr, c.a_qk_norm ? f(MI355_HW_A_KNORM) : nullptr,
-                                          WL.cos_t, WL.sin_t, positions, slot_mapping, T, c.a_heads, c.a_kv_heads, c.a_dim, c.a_vdim,
-                                          c.a_rot_dims, eps, dt, stream));
-            HCHECK(mi355_hyb_window_attention(m->mix, dt, L.out_k, 0, m->q, L.k_pages, L.v_pages, block_tables, context_lens, cu_seqlens_q,
+            const int norm_mode = c.a_qk_norm ? (c.a_norm_after_rot ? 2 : 1) : 0;
+            HCHECK(mi355_hyb_attn_prepare_ex(m->q, L.k_pages, L.v_pages, m->proj, ldp, L.off[P_AQ], L.off[P_AK], L.off[P_AV],
+                                             norm_mode == 1 ? f(MI355_HW_A_QNORM) : nullptr, norm_mode == 1 ? f(MI355_HW_A_KNORM) : nullptr,
+                                             WL.cos_t, WL.sin_t, positions, slot_mapping, T, c.a_heads, c.a_kv_heads, c.a_dim, c.a_vdim,
+                                             c.a_rot_dims, c.a_rot_interleaved, norm_mode, c.a_head_temp ? f(MI355_HW_A_TEMP) : nullptr, eps,
+                                             dt, stream));
+            HCHECK(mi355_hyb_masked_attention(m->mix, dt, L.out_k, 0, m->q, L.k_pages, L.v_pages, block_tables, context_lens, cu_seqlens_q,
                                               m->tok_seq, c.a_has_sink ? f(MI355_HW_A_SINK) : nullptr, num_seqs, T, c.a_heads,
-                                              c.a_kv_heads, c.a_dim, c.a_vdim, m->cfg.block_size, max_blocks, c.a_window, c.a_scale,
-                                              c.mixer == MI355_HYB_MIX_PARALLEL ? c.a_out_scale : 1.f, dt, stream));
+                                              c.a_kv_heads, c.a_dim, c.a_vdim, m->cfg.block_size, max_blocks, c.a_window, c.a_keep_first,
+                                              c.a_scale, c.mixer == MI355_HYB_MIX_PARALLEL ? c.a_out_scale : 1.f, 0, 0, 0.f, 0, dt, stream));
             mix_col = c.a_heads * c.a_vdim;
         }
         if (L.is_latent()) {
@@ -534,12 +599,37 @@ static int forward_enqueue(HModel* m, const uint32_t* tokens, const int64_t* pos
                                     context_lens, cu_seqlens_q, state_slots, num_seqs, T, c.g_width, stream));
         auto residual = [&](int norm_slot) -> int {
             if (m->cfg.residual_form == 1)
-                return mi355_hyb_resid_norm(m->x, bf ? m->xcopy : nullptr, m->y, W, f(norm_slot), T, W, m->cfg.norm_groups, m->cfg.resid_alpha, eps, stream);
-            return mi355_hyb_norm_add(m->x, bf ? m->xcopy : nullptr, m->y, W, f(norm_slot), T, W, eps, stream);
+                return mi355_hyb_resid_norm(m->x, xcopy, m->y, W, f(norm_slot), T, W, m->cfg.norm_groups, m->cfg.resid_alpha, eps, stream);
+            return mi355_hyb_norm_add(m->x, xcopy, m->y, W, f(norm_slot), T, W, eps, stream);
         };
         HCHECK(mi355_hyb_linear(m->y, W, m->mix, dt, L.out_k, WL.w[MI355_HW_OUT_PROJ].p, nullptr, T, W, L.out_k, dt, stream));
         HCHECK(residual(MI355_HW_NORM1));
-        if (c.mlp_kind) {
+        if (c.mlp_kind == 3) {
+            // mixture of experts: route (with the norm in front of it in form 2), group the (token, expert) pairs into whole blocks per
+            // expert, one grouped product for all gate/up matrices, silu, one for all down matrices; the shared expert as dense
+            // products; the weighted sum, the shared expert's gate and the output norm in one launch
+            const int E = c.moe_experts, K = c.moe_top, ff = c.mlp_ff, fs = c.moe_shared_ff, pairs = T * K;
+            const float* router = f(MI355_HW_MOE_ROUTER);
+            HCHECK(mi355_hyb_moe_route(m->moe_ids, m->moe_wts, m->moe_sgate, sandwich ? m->pre : nullptr, dt, m->x,
+                                       sandwich ? f(MI355_HW_PRE_NORM2) : nullptr, router, f(MI355_HW_MOE_CORRECTION),
+                                       fs ? router + (size_t)E * W : nullptr, T, W, E, K, c.moe_scale, eps, stream));
+            const int bm = std::min(mi355_hyb_moe_block_rows(pairs, E, 2 * ff, W, dt), mi355_hyb_moe_block_rows(pairs, E, W, ff, dt));
+            const int nb = (pairs + bm - 1) / bm + E;
+            HCHECK(mi355_hyb_moe_group(m->moe_pos, m->moe_row_token, m->moe_table, m->moe_ids, pairs, K, E, bm, nb, stream));
+            HCHECK(mi355_hyb_linear_grouped(m->moe_gu, 2 * ff, xin, xin_dt, W, m->moe_row_token, WL.w[MI355_HW_MOE_GATE_UP].p, (int64_t)2 * ff * W,
+                                            m->moe_table, bm, nb, 2 * ff, W, dt, stream));
+            HCHECK(mi355_hyb_silu_glu(m->moe_act, dt, m->moe_gu, nb * bm, ff, m->moe_table, bm, stream));
+            HCHECK(mi355_hyb_linear_grouped(m->moe_y, W, m->moe_act, dt, ff, nullptr, WL.w[MI355_HW_MOE_DOWN].p, (int64_t)W * ff, m->moe_table, bm,
+                                            nb, W, ff, dt, stream));
+            if (fs) {
+                HCHECK(mi355_hyb_linear(m->gu, 2 * fs, xin, xin_dt, W, WL.w[MI355_HW_MLP_GATE_UP].p, nullptr, T, 2 * fs, W, dt, stream));
+                HCHECK(mi355_hyb_silu_glu(m->act, dt, m->gu, T, fs, nullptr, 0, stream));
+                HCHECK(mi355_hyb_linear(m->y, W, m->act, dt, fs, WL.w[MI355_HW_MLP_DOWN].p, nullptr, T, W, fs, dt, stream));
+            }
+            HCHECK(mi355_hyb_moe_combine_norm_add(m->x, xcopy, m->moe_y, m->moe_pos, m->moe_wts, fs ? m->y : nullptr, fs ? m->moe_sgate : nullptr,
+                                                  f(MI355_HW_NORM2), T, W, K, eps, stream));
+        } else if (c.mlp_kind) {
+            if (sandwich) HCHECK(mi355_hyb_pre_norm(m->pre, dt, m->x, f(MI355_HW_PRE_NORM2), T, W, eps, stream));
             HCHECK(mi355_hyb_linear(m->gu, 2 * c.mlp_ff, xin, xin_dt, W, WL.w[MI355_HW_MLP_GATE_UP].p, nullptr, T, 2 * c.mlp_ff, W, dt, stream));
             if (c.mlp_kind == 2) HCHECK(mi355_hyb_gelu_glu(m->act, dt, m->gu, T, c.mlp_ff, stream));
             else HCHECK(mi355_hyb_clamped_glu(m->act, dt, m->gu, T, c.mlp_ff, c.mlp_limit, c.mlp_alpha, stream));
@@ -553,6 +643,8 @@ static int forward_enqueue(HModel* m, const uint32_t* tokens, const int64_t* pos
         HCHECK(mi355_hyb_gather_group_norm(m->xn, dt, m->x, out_rows, static_cast<const float*>(m->final_norm.p), n_out, W,
                                            m->cfg.norm_groups, eps, stream));
         HCHECK(mi355_hyb_linear(logits, m->cfg.vocab, m->xn, dt, W, m->head.p, nullptr, n_out, m->cfg.vocab, W, dt, stream));
+        if (m->cfg.logit_scale != 0.f && m->cfg.logit_scale != 1.f)
+            HCHECK(mi355_hyb_scale_f32(logits, m->cfg.logit_scale, (int64_t)n_out * m->cfg.vocab, stream));
     }
     return 0;
 }

@@ -1,6 +1,7 @@
 """Python harness over the `mi355_hybrid_*` handle (include/mi355_hybrid.h): layer-list models whose layers mix tokens by
 sliding-window attention with a sink, a gated delta rule, a minGRU, attention and delta rule side by side, latent attention, or
-attention behind a short convolution with mixed head weights.  The Sogodra and Vivazen designs are read here: a design's
+attention behind a short convolution with mixed head weights, with dense or mixture-of-experts feed-forwards.  The Sogodra, Vivazen
+and Kerolorn designs are read here: a design's
 config.json (`architecture`, `layers`, `norm`, `vocab`, `width`, ...) becomes the C structs, its tensors are concatenated into the
 host layer's slots.  No CPU fallback; torch only holds device buffers."""
 import ctypes
@@ -20,8 +21,9 @@ GATE_SILU, GATE_SIGMOID_LR = 0, 1
 ROPE_DEFAULT, ROPE_LLAMA3, ROPE_YARN = 0, 2, 4
 (HW_EMBED, HW_FINAL_NORM, HW_HEAD, HW_NORM1, HW_NORM2, HW_IN_PROJ, HW_IN_BIAS, HW_OUT_PROJ, HW_A_QNORM, HW_A_KNORM, HW_A_SINK, HW_D_CONV,
  HW_D_A_LOG, HW_D_DT_BIAS, HW_D_NORM, HW_D_A2, HW_D_G2, HW_MLP_GATE_UP, HW_MLP_DOWN, HW_A_CONV, HW_A_TALK, HW_L_UKT, HW_L_UV,
- HW_L_CNORM) = range(24)
-MLP_CLAMPED_GLU, MLP_GELU_GLU = 1, 2
+ HW_L_CNORM, HW_PRE_NORM1, HW_PRE_NORM2, HW_IN_CONV, HW_A_TEMP, HW_MOE_ROUTER, HW_MOE_CORRECTION, HW_MOE_GATE_UP,
+ HW_MOE_DOWN) = range(32)
+MLP_CLAMPED_GLU, MLP_GELU_GLU, MLP_MOE = 1, 2, 3
 
 # constants the Sogodra design fixes
 SOGODRA_GLU_ALPHA = 1.702          # y = g sigmoid(1.702 g) (u + 1)
@@ -82,6 +84,22 @@ class HeadTranspose:
         rows, cols = shapes[self.name]
         a = np.asarray(bits[self.name], np.uint16).reshape(self.heads, rows // self.heads, cols)
         return np.ascontiguousarray(a.transpose(0, 2, 1)).reshape(-1)
+
+
+def yarn_scaling(rot):
+    """`rot.scaling` = {factor, original, fast, slow} -> the table builder's yarn form: the frequency blend between the indices where a
+    wavelength makes `fast` / `slow` turns over `original` positions, amplitude 0.1 ln(factor) + 1 on cos and sin for EVERY factor (the
+    table builder keeps amplitude 1 up to factor 1, so there it is passed as the attention factor)"""
+    rs = RopeScaling()
+    sc = rot.get("scaling")
+    if sc:
+        rs.type, rs.factor, rs.original_max_position_embeddings = ROPE_YARN, float(sc["factor"]), float(sc["original"])
+        rs.beta_fast, rs.beta_slow, rs.attn_factor = float(sc["fast"]), float(sc["slow"]), 1.0
+        if rs.factor <= 1.0:
+            rs.attn_factor = 0.1 * math.log(rs.factor) + 1.0
+    else:
+        rs.type = ROPE_DEFAULT
+    return rs
 
 
 class SogodraSpec:
@@ -181,18 +199,7 @@ class VivazenSpec:
     `weights_of` runs on that layer's tensors with a cache of its own."""
     residual_form = 1
 
-    @staticmethod
-    def rope_scaling(rot):
-        rs = RopeScaling()
-        sc = rot.get("scaling")
-        if sc:
-            rs.type, rs.factor, rs.original_max_position_embeddings = ROPE_YARN, float(sc["factor"]), float(sc["original"])
-            rs.beta_fast, rs.beta_slow, rs.attn_factor = float(sc["fast"]), float(sc["slow"]), 1.0
-            if rs.factor <= 1.0:              # the table builder keeps amplitude 1 up to factor 1; this design's 0.1 ln(factor) + 1 holds for every factor
-                rs.attn_factor = 0.1 * math.log(rs.factor) + 1.0
-        else:
-            rs.type = ROPE_DEFAULT
-        return rs
+    rope_scaling = staticmethod(yarn_scaling)
 
     def __init__(self, cfg, shapes):
         if cfg.get("architecture") != "Vivazen":
@@ -258,7 +265,75 @@ class VivazenSpec:
         return L, slots, rope
 
 
-SPECS = {"Sogodra": SogodraSpec, "Vivazen": VivazenSpec}       # config.json `architecture` -> its reader
+class KerolornSpec:
+    """config.json of a Kerolorn model -> layer structs + the tensor names behind every weight slot.  The design: a norm on both sides
+    of every sublayer, x <- x + Nb(sub(Na(x))); the mixer's input h becomes h + conv(h) (`canon1`, a causal convolution over time per
+    channel of the width); grouped-query attention with interleaved rotary pairs (yarn), a weightless RMS norm of q and k behind the
+    rotation, a temperature per head, a sliding window that keeps the first tokens; mixture-of-experts feed-forward (softmax router,
+    selection-only correction, scaled weights, shared expert behind a sigmoid gate); logits times `logit_scale`."""
+    residual_form, resid_alpha, norm_groups = 2, 1.0, 1
+    rope_scaling = staticmethod(yarn_scaling)
+
+    def __init__(self, cfg, shapes):
+        if cfg.get("architecture") != "Kerolorn":
+            raise ValueError("not a Kerolorn config")
+        self.cfg = cfg
+        self.width, self.vocab = int(cfg["width"]), int(cfg["vocab"])
+        self.eps = float(cfg["norm"]["eps"])
+        self.logit_scale = float(cfg.get("logit_scale", 1.0))
+        self.taps = int((cfg.get("canon") or {}).get("taps", 0))
+        self.layers, self.slots, self.rope = [], [], []
+        for i, lc in enumerate(cfg["layers"]):
+            L, slots, rope = self._layer("l%d." % i, lc, shapes)
+            self.layers.append(L)
+            self.slots.append(slots)
+            self.rope.append(rope)
+
+    def _layer(self, p, lc, shapes):
+        if lc["type"] != "attention":
+            raise ValueError(f"layer type {lc['type']!r} is not part of the design")
+        L, c, q = HybridLayer(), lc["mixer"], p + "mix."
+        slots = {HW_PRE_NORM1: [p + "norm1"], HW_NORM1: [p + "norm1b"]}
+        L.mixer = MIX_ATTENTION
+        L.a_heads, L.a_kv_heads, L.a_dim, L.a_vdim = int(c["heads"]), int(c["kv_heads"]), int(c["dim"]), int(c["vdim"])
+        L.a_scale, L.a_out_scale = float(c["scale"]), 1.0
+        mask = c.get("mask") or {}
+        L.a_window, L.a_keep_first = int(mask.get("size") or 0), int(mask.get("keep_first") or 0)
+        rope = c.get("rot")
+        L.a_rot_dims, L.a_rot_interleaved = (int(rope["dims"]) if rope else 0), 1
+        if L.a_rot_dims <= 0:
+            rope = None
+        L.a_qk_norm, L.a_norm_after_rot = 1, 1
+        L.a_head_temp = int(q + "temp" in shapes)
+        if L.a_head_temp:
+            slots[HW_A_TEMP] = [q + "temp"]
+        if p + "canon1" in shapes:
+            L.in_conv = int(shapes[p + "canon1"][1])
+            if self.taps and L.in_conv != self.taps:
+                raise ValueError(f"{p}canon1 has {L.in_conv} taps, the config says {self.taps}")
+            slots[HW_IN_CONV] = [p + "canon1"]
+        slots[HW_IN_PROJ], slots[HW_OUT_PROJ] = [q + "q", q + "k", q + "v"], [q + "o"]
+        mlp = lc.get("mlp")
+        if mlp:
+            if mlp.get("kind", "moe") != "moe":
+                raise ValueError(f"feed-forward kind {mlp.get('kind')!r} is not part of the design")
+            m, r = p + "mlp.", mlp["router"]
+            L.mlp_kind, L.mlp_ff = MLP_MOE, int(mlp["expert"]["ff"])
+            L.moe_experts, L.moe_top, L.moe_scale = int(r["experts"]), int(r["top"]), float(r.get("scale", 1.0))
+            shared = mlp.get("shared")
+            L.moe_shared_ff = int(shared["ff"]) if shared else 0
+            slots[HW_PRE_NORM2], slots[HW_NORM2] = [p + "norm2"], [p + "norm2b"]
+            slots[HW_MOE_ROUTER] = [m + "router"] + ([m + "shared.sg"] if shared else [])
+            if m + "correction" in shapes:
+                slots[HW_MOE_CORRECTION] = [m + "correction"]
+            slots[HW_MOE_GATE_UP] = [m + "e%d.%s" % (e, n) for e in range(L.moe_experts) for n in ("gate", "up")]
+            slots[HW_MOE_DOWN] = [m + "e%d.down" % e for e in range(L.moe_experts)]
+            if shared:
+                slots[HW_MLP_GATE_UP], slots[HW_MLP_DOWN] = [m + "shared.gate", m + "shared.up"], [m + "shared.down"]
+        return L, slots, rope
+
+
+SPECS = {"Sogodra": SogodraSpec, "Vivazen": VivazenSpec, "Kerolorn": KerolornSpec}       # config.json `architecture` -> its reader
 
 
 class HybridModel:
@@ -272,7 +347,8 @@ class HybridModel:
         self._layers = (HybridLayer * n)(*spec.layers)
         c = HybridConfig(width=spec.width, vocab=spec.vocab, n_layers=n, dtype=self.dtype, block_size=self.block_size,
                          state_slots=self.state_slots, norm_eps=spec.eps, unit_eps=SOGODRA_UNIT_EPS,
-                         residual_form=int(spec.residual_form), resid_alpha=float(spec.resid_alpha), norm_groups=int(spec.norm_groups))
+                         residual_form=int(spec.residual_form), resid_alpha=float(spec.resid_alpha), norm_groups=int(spec.norm_groups),
+                         logit_scale=float(getattr(spec, "logit_scale", 1.0)))
         self.h = lib.mi355_hybrid_create(ctypes.byref(c), self._layers)
         if not self.h:
             raise RuntimeError("mi355_hybrid_create refused the configuration")

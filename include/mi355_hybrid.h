@@ -1,8 +1,8 @@
 /* C ABI of the layer-list ("hybrid") host layer: decoder-only models whose config lists, layer by layer, which token mixer a
  * layer has -- sliding-window attention with a softmax sink, a gated delta rule (recurrent matrix state), a minGRU (recurrent vector
  * state), attention and delta rule side by side, latent attention (keys and values read off one cached latent vector per token), or
- * attention behind a short convolution whose heads' softmax weights are mixed -- and which feed-forward.  The Sogodra and Vivazen
- * designs are its users.
+ * attention behind a short convolution whose heads' softmax weights are mixed -- and which feed-forward (dense gate/up forms or a
+ * mixture of experts).  The Sogodra, Vivazen and Kerolorn designs are its users.
  *
  * What differs from the llama-family host layers (mi355_llama_*, mi355_dense_*):
  *   - the residual stream, norms, attention scores, decays, gates of a recurrence and the recurrent state are f32 in both dtypes;
@@ -55,7 +55,9 @@ typedef struct mi355_hybrid_layer {
     /* minGRU */
     int32_t g_width;
     /* feed-forward: 0 = none, 1 = dense clamped gate/up with y = g sigmoid(act_alpha g) (u + 1),
-                     2 = dense gate/up with y = gelu_tanh(g) u                                                     */
+                     2 = dense gate/up with y = gelu_tanh(g) u,
+                     3 = mixture of experts with y = silu(g) u (fields below; the shared expert, when there is one, uses the dense
+                         slots MI355_HW_MLP_GATE_UP / _DOWN with moe_shared_ff)                                       */
     int32_t mlp_kind, mlp_ff;
     float mlp_limit, mlp_alpha;
     /* more switches of the attention branch (all 0 = the plain form) */
@@ -71,6 +73,18 @@ typedef struct mi355_hybrid_layer {
                                       weights to the values of its own key/value head                                      */
     int32_t share_with;            /* 0: the layer has weights; n > 0: it runs on layer n - 1's weights (and rope tables) with
                                       pages and state of its own                                                           */
+    /* switches of the plain attention mixers (MI355_HYB_MIX_ATTENTION / _PARALLEL), all 0 = the form above */
+    int32_t a_keep_first;          /* with a window: keys at positions < a_keep_first stay visible to every later query     */
+    int32_t a_norm_after_rot;      /* the RMS norm of q and k (a_qk_norm) is taken AFTER the rotation and has no weight     */
+    int32_t a_head_temp;           /* head h's scores are multiplied by temp[h] (MI355_HW_A_TEMP)                           */
+    /* input convolution in front of the mixer: what the mixer reads, h, becomes h + conv(h), a causal convolution over time on
+     * every channel of the width (in_conv taps, 0 = none); the last taps - 1 rows of h live in the state slot                  */
+    int32_t in_conv;
+    /* feed-forward kind 3, a mixture of experts: moe_experts gate/up experts of mlp_ff with silu, every token uses the moe_top with
+     * the largest softmax(router) + correction; its weights are the chosen experts' softmax values times moe_scale (not
+     * renormalised).  moe_shared_ff > 0: one more expert of that size runs for every token, times sigmoid(w_sg . h)              */
+    int32_t moe_experts, moe_top, moe_shared_ff;
+    float moe_scale;
 } mi355_hybrid_layer;
 
 typedef struct mi355_hybrid_config {
@@ -80,10 +94,13 @@ typedef struct mi355_hybrid_config {
     int32_t state_slots;           /* recurrent-state slots (live sequences)                                       */
     float norm_eps;
     float unit_eps;                /* eps inside the root of the unit norm of q and k in the delta rule            */
-    int32_t residual_form;         /* 0: x <- x + norm(sub(x));  1: x <- norm(resid_alpha x + sub(x))                */
+    int32_t residual_form;         /* 0: x <- x + norm(sub(x));  1: x <- norm(resid_alpha x + sub(x));
+                                      2: x <- x + norm(sub(pre_norm(x))), a norm on both sides of every sublayer
+                                         (MI355_HW_PRE_NORM1 / 2 in front, MI355_HW_NORM1 / 2 behind)                 */
     float resid_alpha;
     int32_t norm_groups;           /* the layer norms and the last norm take the RMS over this many equal consecutive parts
                                       of the vector separately (0 or 1: over the whole vector)                       */
+    float logit_scale;             /* the logits are multiplied by it (0 = 1)                                        */
 } mi355_hybrid_config;
 
 /* weight slots: `layer` = -1 for the three global ones */
@@ -112,7 +129,15 @@ typedef struct mi355_hybrid_config {
 #define MI355_HW_L_UKT 21          /* [heads, kv_rank, dim]: per head the TRANSPOSE of its block of W_uk [heads dim, kv_rank] */
 #define MI355_HW_L_UV 22           /* [heads vdim, kv_rank]                                                         */
 #define MI355_HW_L_CNORM 23        /* [kv_rank] weight of the latent's RMS norm                                      */
-#define MI355_HW_COUNT 24
+#define MI355_HW_PRE_NORM1 24      /* [width]  residual form 2: norm in front of the mixer                           */
+#define MI355_HW_PRE_NORM2 25      /* [width]  residual form 2: norm in front of the feed-forward                    */
+#define MI355_HW_IN_CONV 26        /* [width, in_conv], last column = the current token                              */
+#define MI355_HW_A_TEMP 27         /* [heads]                                                                        */
+#define MI355_HW_MOE_ROUTER 28     /* f32 [experts (+ 1 when moe_shared_ff: the shared expert's gate row last), width] */
+#define MI355_HW_MOE_CORRECTION 29 /* [experts] added to the softmax values for the choice only                      */
+#define MI355_HW_MOE_GATE_UP 30    /* [experts, 2 ff, width]: per expert gate rows, then up rows                     */
+#define MI355_HW_MOE_DOWN 31       /* [experts, width, ff]                                                           */
+#define MI355_HW_COUNT 32
 
 void* mi355_hybrid_create(const mi355_hybrid_config* cfg, const mi355_hybrid_layer* layers);
 void mi355_hybrid_destroy(void* model);
@@ -232,6 +257,62 @@ int mi355_hyb_conv(float* out, const float* proj, int32_t ldp, int32_t off, cons
                    int64_t state_stride, const uint32_t* context_lens, const uint32_t* cu_seqlens_q, const int32_t* state_slots,
                    const int32_t* token_seq, int32_t num_seqs, int32_t num_tokens, int32_t channels, int32_t taps, int32_t act,
                    int64_t stream);
+/* ---- mechanisms of the pre/post-norm designs */
+/* out (dt_out) [T, width] = RMS norm of every row of x times w (the norm in front of a sublayer) */
+int mi355_hyb_pre_norm(void* out, int32_t out_dtype, const float* x, const float* w, int32_t num_tokens, int32_t width, float eps,
+                       int64_t stream);
+/* out (dt_out) [T, channels] = h + conv(h) for h = in f32 [T, ld] columns [off, off + channels): the causal convolution of
+ * mi355_hyb_conv added to its own input; mi355_hyb_conv_state_update(in) then moves the state behind the portion */
+int mi355_hyb_conv_residual(void* out, int32_t out_dtype, const float* in, int32_t ld, int32_t off, const float* w,
+                            const float* conv_state, int64_t state_stride, const uint32_t* context_lens, const uint32_t* cu_seqlens_q,
+                            const int32_t* state_slots, const int32_t* token_seq, int32_t num_seqs, int32_t num_tokens, int32_t channels,
+                            int32_t taps, int64_t stream);
+/* mi355_hyb_attn_prepare with the remaining switches: interleaved = rotated pairs are (2i, 2i + 1); norm_mode 0 = none, 1 = RMS norm
+ * with weights before the rotation (q_norm_w / k_norm_w, NULL = no weight), 2 = RMS norm without a weight AFTER the rotation;
+ * q_head_scale f32 [heads] or NULL: head h's query is multiplied by it (a temperature per head folded into the query) */
+int mi355_hyb_attn_prepare_ex(void* q_out, void* k_pages, void* v_pages, const float* proj, int32_t ldp, int32_t q_off, int32_t k_off,
+                              int32_t v_off, const float* q_norm_w, const float* k_norm_w, const float* cos_t, const float* sin_t,
+                              const int64_t* positions, const int64_t* slot_mapping, int32_t num_tokens, int32_t heads,
+                              int32_t kv_heads, int32_t dim, int32_t vdim, int32_t rot_dims, int32_t interleaved, int32_t norm_mode,
+                              const float* q_head_scale, float eps, int32_t dtype, int64_t stream);
+/* mi355_hyb_window_attention_ex with kept first tokens: a query at position i sees key j when j <= i and (window == 0 or
+ * i - j < window or j < keep_first); kept keys keep their own positions */
+int mi355_hyb_masked_attention(void* out, int32_t out_dtype, int32_t ldo, int32_t out_off, const void* q, const void* k_pages,
+                               const void* v_pages, const uint32_t* block_tables, const uint32_t* context_lens,
+                               const uint32_t* cu_seqlens_q, const int32_t* token_seq, const float* sink, int32_t num_seqs,
+                               int32_t num_tokens, int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, int32_t block_size,
+                               int32_t max_blocks, int32_t window, int32_t keep_first, float scale, float out_scale, int32_t k_ld,
+                               int32_t v_ld, float softcap, int32_t cross_values, int32_t dtype, int64_t stream);
+/* mixture of experts, routing: h = RMS norm of x times norm_w (norm_w NULL: h = x) -> xn (dt_out) [T, width] (NULL = not written);
+ * z = router f32 [experts, width] . h in f32, s = softmax(z); the `top` experts with the largest s + correction (correction NULL =
+ * none; ties to the lower expert) -> expert_ids i32 [T, top] in descending order of the choice score, weights f32 [T, top] =
+ * s[chosen] * scale.  gate_row f32 [width] or NULL: shared_gate f32 [T] = sigmoid(gate_row . h) */
+int mi355_hyb_moe_route(int32_t* expert_ids, float* weights, float* shared_gate, void* xn, int32_t out_dtype, const float* x,
+                        const float* norm_w, const float* router, const float* correction, const float* gate_row, int32_t num_tokens,
+                        int32_t width, int32_t experts, int32_t top, float scale, float eps, int64_t stream);
+/* rows of a grouped product's blocks that suit `pairs` (token, expert) pairs over `experts` experts with [n, k] matrices: 16 (few
+ * rows per expert: a stream over the weights), 64 or 128 (matrix-core tiles through LDS) */
+int32_t mi355_hyb_moe_block_rows(int32_t pairs, int32_t experts, int32_t n, int32_t k, int32_t dtype);
+/* grouping on the device: every expert owns whole blocks of block_rows rows of the gathered buffers, expert e's rows start at
+ * block_rows * (blocks of the experts before it).  pos i32 [pairs] = the row of pair p = token * top + slot; row_token i32 [n_blocks *
+ * block_rows] = the token of every used row; block_table i32 [n_blocks, 2] = {expert, one past the expert's last row} for every block
+ * ({0, 0} past the last expert's), n_blocks >= ceil(pairs / block_rows) + experts */
+int mi355_hyb_moe_group(int32_t* pos, int32_t* row_token, int32_t* block_table, const int32_t* expert_ids, int32_t pairs, int32_t top,
+                        int32_t experts, int32_t block_rows, int32_t n_blocks, int64_t stream);
+/* one product per block of the table: out f32 rows [b block_rows, block end) = a rows . (w + expert w_bs) [n, k]^T; a (dt_a) [.., lda]
+ * row r is read at row_token[r] when row_token != NULL (gathered from the token rows), else at r */
+int mi355_hyb_linear_grouped(float* out, int32_t ldo, const void* a, int32_t a_dtype, int32_t lda, const int32_t* row_token,
+                             const void* w, int64_t w_bs, const int32_t* block_table, int32_t block_rows, int32_t n_blocks, int32_t n,
+                             int32_t k, int32_t dtype, int64_t stream);
+/* out (dt_out) [rows, ff] = silu(gu[:, j]) gu[:, ff + j]; block_table != NULL: only the rows that a block of the table uses */
+int mi355_hyb_silu_glu(void* out, int32_t out_dtype, const float* gu, int32_t rows, int32_t ff, const int32_t* block_table,
+                       int32_t block_rows, int64_t stream);
+/* x f32 [T, width] += y / rms(y) * w with y[t] = sum_j weights[t, j] y_rows[pos[t top + j]] + shared_gate[t] y_shared[t]
+ * (y_shared NULL = no shared expert; shared_gate NULL = 1); xcopy: NULL or bf16 [T, width] */
+int mi355_hyb_moe_combine_norm_add(float* x, void* xcopy, const float* y_rows, const int32_t* pos, const float* weights,
+                                   const float* y_shared, const float* shared_gate, const float* w, int32_t num_tokens, int32_t width,
+                                   int32_t top, float eps, int64_t stream);
+int mi355_hyb_scale_f32(float* x, float s, int64_t n, int64_t stream);
 /* 0: prompt-sized steps over bf16 pages take the generic kernel instead of the matrix-core one (A/B switch, process-wide; default 1) */
 void mi355_hyb_set_attention_mfma(int32_t on);
 /* short causal convolution over time per channel, then silu: out f32 [T, channels] from proj columns [off, off + channels);
