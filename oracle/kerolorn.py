@@ -63,13 +63,18 @@ def head_temperature_attention(q, k, v, q_pos, k_pos, scale, temp, window=0, kee
 
 
 # ---------------------------------------------------------------------------------------------------------------- mixture of experts
-def route(h, w_router, correction, top, scale):
+def route(h, w_router, correction, top, scale, margins=None):
     """h [T, W] -> (chosen experts [T, top] by descending choice score, weights [T, top]).  s = softmax(W_r h); the choice is made on
-    s + correction, the weight of a chosen expert is its s times `scale` (no renormalisation)"""
+    s + correction, the weight of a chosen expert is its s times `scale` (no renormalisation).  margins: a list that receives, per
+    token, the gap between the last chosen and the first rejected choice score (how close the call was)"""
     z = h @ w_router.T
     e = np.exp(z - z.max(axis=1, keepdims=True))
     s = e / e.sum(axis=1, keepdims=True)
-    order = np.argsort(-(s + correction), axis=1, kind="stable")[:, :top]
+    choice = s + correction
+    order = np.argsort(-choice, axis=1, kind="stable")[:, :top]
+    if margins is not None and top < choice.shape[1]:
+        ranked = -np.sort(-choice, axis=1)
+        margins.extend((ranked[:, top - 1] - ranked[:, top]).tolist())
     return order, np.take_along_axis(s, order, axis=1) * scale
 
 
@@ -77,9 +82,10 @@ def silu_expert(h, gate, up, down):
     return (silu(h @ gate.T) * (h @ up.T)) @ down.T
 
 
-def moe(h, W, p, n_experts, top, scale, shared):
+def moe(h, W, p, n_experts, top, scale, shared, margins=None):
     """W: name -> array, p: the feed-forward's prefix ('l3.mlp.')"""
-    idx, wt = route(h, W[p + "router"], W[p + "correction"], top, scale)
+    corr = W[p + "correction"] if p + "correction" in W else np.zeros(n_experts)
+    idx, wt = route(h, W[p + "router"], corr, top, scale, margins)
     y = np.zeros((h.shape[0], W[p + "e0.down"].shape[0]))
     for e in range(n_experts):
         for t, k in zip(*np.nonzero(idx == e)):
@@ -104,6 +110,7 @@ class KerolornOracle:
     def reset(self):
         self.pos = 0
         self.state = [dict() for _ in self.cfg["layers"]]
+        self.margins = []             # of every routing decision so far (route)
 
     def _attention(self, st, p, c, h, positions):
         W = self.W
@@ -120,7 +127,8 @@ class KerolornOracle:
         st["k"] = k if "k" not in st else np.concatenate([st["k"], k])
         st["v"] = v if "v" not in st else np.concatenate([st["v"], v])
         mask = c.get("mask") or {}
-        o = head_temperature_attention(q, st["k"], st["v"], positions, list(range(len(st["k"]))), c["scale"], W[p + "temp"],
+        o = head_temperature_attention(q, st["k"], st["v"], positions, list(range(len(st["k"]))), c["scale"],
+                                       W[p + "temp"] if p + "temp" in W else np.ones(H),
                                        int(mask.get("size", 0)), int(mask.get("keep_first", 0)))
         return o.reshape(T, H * vd) @ W[p + "o"].T
 
@@ -143,7 +151,7 @@ class KerolornOracle:
             if mlp:
                 h = rms_norm(x, W[p + "norm2"], self.eps)
                 r = mlp["router"]
-                y = moe(h, W, p + "mlp.", r["experts"], r["top"], r["scale"], bool(mlp.get("shared")))
+                y = moe(h, W, p + "mlp.", r["experts"], r["top"], r["scale"], bool(mlp.get("shared")), self.margins)
                 x = x + rms_norm(y, W[p + "norm2b"], self.eps)
             trace.append(x.copy())
         return rms_norm(x, W["final.norm"], self.eps) @ W["head"].T * cfg.get("logit_scale", 1.0), np.stack(trace)
@@ -181,7 +189,7 @@ def random_kerolorn(rng, cfg, scale=1.0):
             for e in range(E):
                 mat(m + "e%d.gate" % e, ff, Wd); mat(m + "e%d.up" % e, ff, Wd); mat(m + "e%d.down" % e, Wd, ff)
             mat(m + "router", E, Wd, 2.0 / math.sqrt(Wd))
-            vec(m + "correction", E, 0.0, 0.05)
+            W[m + "correction"] = bf16_round(rng.uniform(0.0, 2.0 / E, E))       # of the softmax values' size: both decide the choice
             if mlp.get("shared"):
                 fs = mlp["shared"]["ff"]
                 mat(m + "shared.gate", fs, Wd); mat(m + "shared.up", fs, Wd); mat(m + "shared.down", Wd, fs)
