@@ -1,5 +1,5 @@
-"""`python bench.py --hybrid`: prompt and decode throughput of the layer-list host layer (Sogodra design, or Vivazen with
-`--hybrid-design vivazen`; random weights) at layer sizes of a real model, beside the framework's closest existing model -- the 16-bit llama host layer (dense_model.cpp) -- at equal
+"""`python bench.py --hybrid`: prompt and decode throughput of the layer-list host layer (Sogodra design, or Vivazen / Kerolorn with
+`--hybrid-design vivazen|kerolorn`; random weights) at layer sizes of a real model, beside the framework's closest existing model -- the 16-bit llama host layer (dense_model.cpp) -- at equal
 width, depth, head geometry, feed-forward size and vocabulary.  One GPU, bf16, synthetic data.  The default workload of bench.py and
 its one-line contract are not touched: this option prints its own JSON line.
 
@@ -26,6 +26,44 @@ VIVAZEN = {
     "3b": dict(l_heads=24, l_dim=64, l_rot=64, l_rank=192, l_vdim=64, taps=4, layers="laal"),
     "8b": dict(l_heads=32, l_dim=128, l_rot=64, l_rank=192, l_vdim=128, taps=4, layers="laal"),
 }
+
+
+# Kerolorn at the same widths: attention with the llama geometry (window, kept first tokens, rotation on half of the head), input
+# convolution, and a mixture of experts whose ACTIVE size equals the llama feed-forward: `top` experts + the shared one, each ff / 4
+KEROLORN = {
+    "1b": dict(experts=16, top=3, keep=64, taps=4, layers=4),
+    "3b": dict(experts=16, top=3, keep=64, taps=4, layers=4),
+    "8b": dict(experts=16, top=3, keep=64, taps=4, layers=4),
+}
+
+
+def kerolorn_config(s, v):
+    att = {"dim": s["dim"], "heads": s["heads"], "kv_heads": s["kv"], "vdim": s["dim"], "scale": 1.2 * s["dim"] ** -0.5,
+           "mask": {"size": s["window"], "keep_first": v["keep"]},
+           "rot": {"base": 500000.0, "dims": s["dim"] // 2, "scaling": {"factor": 4.0, "fast": 24.0, "original": 4096, "slow": 2.0}}}
+    mlp = {"expert": {"ff": s["ff"] // 4}, "kind": "moe", "router": {"experts": v["experts"], "scale": 2.0, "top": v["top"]},
+           "shared": {"ff": s["ff"] // 4}}
+    return {"architecture": "Kerolorn", "canon": {"taps": v["taps"]}, "layers": [{"type": "attention", "mixer": att, "mlp": mlp}] * v["layers"],
+            "logit_scale": 1.5, "norm": {"eps": 1e-6}, "vocab": s["vocab"], "width": s["width"]}
+
+
+def kerolorn_shapes(cfg):
+    W, sh = cfg["width"], {}
+    sh["embed"], sh["final.norm"], sh["head"] = (cfg["vocab"], W), (W,), (cfg["vocab"], W)
+    for i, lc in enumerate(cfg["layers"]):
+        p, c, mlp = "l%d." % i, lc["mixer"], lc["mlp"]
+        q, m = p + "mix.", p + "mlp."
+        for n in ("norm1", "norm1b", "norm2", "norm2b"):
+            sh[p + n] = (W,)
+        sh[p + "canon1"] = (W, cfg["canon"]["taps"])
+        H, G, d, vd = c["heads"], c["kv_heads"], c["dim"], c["vdim"]
+        sh[q + "q"], sh[q + "k"], sh[q + "v"], sh[q + "temp"], sh[q + "o"] = (H * d, W), (G * d, W), (G * vd, W), (H,), (W, H * vd)
+        ff, E, fs = mlp["expert"]["ff"], mlp["router"]["experts"], mlp["shared"]["ff"]
+        for e in range(E):
+            sh[m + "e%d.gate" % e], sh[m + "e%d.up" % e], sh[m + "e%d.down" % e] = (ff, W), (ff, W), (W, ff)
+        sh[m + "router"], sh[m + "correction"] = (E, W), (E,)
+        sh[m + "shared.gate"], sh[m + "shared.up"], sh[m + "shared.down"], sh[m + "shared.sg"] = (fs, W), (fs, W), (W, fs), (1, W)
+    return sh
 
 
 def vivazen_config(s, v):
@@ -118,7 +156,7 @@ def build_hybrid(cfg, max_tokens, slots):
     """random weights generated on the GPU, concatenated as the loader does it, handed over as device bf16"""
     import torch
     from candle_vllm_amd import hybrid_model as hm
-    shapes = vivazen_shapes(cfg) if cfg["architecture"] == "Vivazen" else sogodra_shapes(cfg)
+    shapes = {"Vivazen": vivazen_shapes, "Kerolorn": kerolorn_shapes, "Sogodra": sogodra_shapes}[cfg["architecture"]](cfg)
     spec = hm.SPECS[cfg["architecture"]](cfg, shapes)
     m = hm.HybridModel(spec, dtype="bfloat16", block_size=64, state_slots=slots)
     g = torch.Generator(device="cuda").manual_seed(7)
@@ -126,13 +164,17 @@ def build_hybrid(cfg, max_tokens, slots):
 
     def rnd(shape, name):
         fan = shape[-1] if len(shape) > 1 else 1
-        if name.endswith("norm") or name.endswith("norm1") or name.endswith("norm2"):
+        if name.split(".")[-1].startswith("norm") or name.endswith(".temp"):
             return (1 + 0.02 * torch.randn(shape, generator=g, device="cuda")).to(torch.bfloat16)
+        if name.endswith(".correction"):
+            return (0.05 * torch.rand(shape, generator=g, device="cuda")).to(torch.bfloat16)
+        if name.endswith(".router"):
+            return (2.0 * fan ** -0.5 * torch.randn(shape, generator=g, device="cuda")).to(torch.bfloat16)
         if name == "embed":
             return torch.randn(shape, generator=g, device="cuda").to(torch.bfloat16)
         if name.endswith(".talk"):
             return (torch.eye(shape[0], device="cuda") + 0.1 * torch.randn(shape, generator=g, device="cuda")).to(torch.bfloat16)
-        s = 0.5 if name.endswith(".conv") else (fan ** -0.5 if len(shape) > 1 else 0.3)
+        s = 0.5 if name.endswith(".conv") else 0.3 if name.endswith("canon1") else (fan ** -0.5 if len(shape) > 1 else 0.3)
         return (s * torch.randn(shape, generator=g, device="cuda")).to(torch.bfloat16)
 
     def put(layer, which, names, axis=0):
@@ -172,9 +214,10 @@ def run_size(name, T=2048, B=8, ctx=2048, dec_steps=16, design="sogodra"):
     from candle_vllm_amd.step_engine import StepEngine
     from oracle.dense_llama import DenseConfig
     s = SIZES[name]
-    cfg = vivazen_config(s, VIVAZEN[name]) if design == "vivazen" else sogodra_config(s)
+    extra = {"vivazen": VIVAZEN, "kerolorn": KEROLORN}.get(design, {}).get(name, {})
+    cfg = vivazen_config(s, extra) if design == "vivazen" else kerolorn_config(s, extra) if design == "kerolorn" else sogodra_config(s)
     rng = np.random.default_rng(5)
-    out = {"size": name, "design": design, "shape": dict(s, **(VIVAZEN[name] if design == "vivazen" else {})), "prompt_tokens": T, "decode_batch": B,
+    out = {"size": name, "design": design, "shape": dict(s, **extra), "prompt_tokens": T, "decode_batch": B,
            "decode_ctx": ctx}
     sync = torch.cuda.synchronize
     # ---- hybrid: prompt step, then B sequences decoding behind ctx tokens
@@ -243,8 +286,8 @@ def run_size(name, T=2048, B=8, ctx=2048, dec_steps=16, design="sogodra"):
 
 
 def main(sizes="1b,3b", prompt_tokens=2048, batch=8, ctx=2048, design="sogodra"):
-    if design not in ("sogodra", "vivazen"):
-        raise SystemExit("--hybrid-design: sogodra or vivazen")
+    if design not in ("sogodra", "vivazen", "kerolorn"):
+        raise SystemExit("--hybrid-design: sogodra, vivazen or kerolorn")
     res = [run_size(n.strip(), T=prompt_tokens, B=batch, ctx=ctx, design=design) for n in sizes.split(",") if n.strip()]
     print(json.dumps({"metric": "hybrid_vs_llama_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "n_gpus": 1,
                       "note": "%s layer-list host layer beside the 16-bit llama host layer at equal sizes; the hybrid side's decode steps replay "

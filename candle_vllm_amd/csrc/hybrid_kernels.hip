@@ -1321,14 +1321,14 @@ template <typename TO> __global__ void head_gate_kernel(TO* out, const float* in
 // Routing, one workgroup per token: the normalised row h is built once in LDS (and written out for the experts' products), a wave
 // takes the experts e = wave, wave + 4, ... (f32 router rows . h), then wave 0 makes the softmax, the choice by s + correction
 // (largest first, ties to the lower expert) and the weights s[chosen] * scale.  The shared expert's gate is one more row.
-template <typename TO> __global__ __launch_bounds__(256) void moe_route_kernel(int32_t* ids, float* wts, float* sgate, TO* xn, const float* x,
+template <typename TO, int NW> __global__ __launch_bounds__(64 * NW) void moe_route_kernel(int32_t* ids, float* wts, float* sgate, TO* xn, const float* x,
                                                                                const float* norm_w, const float* router, const float* corr,
                                                                                const float* gate_row, int width, int E, int K, float scale,
                                                                                float eps) {
     extern __shared__ __align__(16) float rsm[];
     float* hs = rsm;                       // [width]
     float* logit = hs + width;             // [E + 1]
-    __shared__ float red[4];
+    __shared__ float red[NW];
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float* xr = x + (size_t)t * width;
     float inv = 1.f;
@@ -1344,13 +1344,21 @@ template <typename TO> __global__ __launch_bounds__(256) void moe_route_kernel(i
     }
     __syncthreads();
     const int rows = E + (gate_row ? 1 : 0);
-    for (int e = wave; e < rows; e += 4) {
+    for (int e = wave; e < rows; e += NW) {
         const float* g = e < E ? router + (size_t)e * width : gate_row;
         float acc = 0.f;
         if ((width & 3) == 0) {
-            for (int i = 4 * lane; i < width; i += 256) {
-                const float4 gv = *reinterpret_cast<const float4*>(g + i), hv = *reinterpret_cast<const float4*>(hs + i);
-                acc = fmaf(hv.x, gv.x, fmaf(hv.y, gv.y, fmaf(hv.z, gv.z, fmaf(hv.w, gv.w, acc))));
+            // eight 16-byte pieces of the row per lane are requested before the first is used
+            for (int i0 = 4 * lane; i0 < width; i0 += 8 * 256) {
+                float4 gv[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) gv[u] = i0 + 256 * u < width ? *reinterpret_cast<const float4*>(g + i0 + 256 * u) : float4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    if (i0 + 256 * u >= width) break;
+                    const float4 hv = *reinterpret_cast<const float4*>(hs + i0 + 256 * u);
+                    acc = fmaf(hv.x, gv[u].x, fmaf(hv.y, gv[u].y, fmaf(hv.z, gv[u].z, fmaf(hv.w, gv[u].w, acc))));
+                }
             }
         } else {
             for (int i = lane; i < width; i += 64) acc = fmaf(hs[i], g[i], acc);
@@ -1432,36 +1440,56 @@ template <typename TO> __global__ void silu_glu_kernel(TO* out, const float* gu,
     st<TO>(out, (size_t)i, siluf_(gu[t * 2 * ff + j]) * gu[t * 2 * ff + ff + j]);
 }
 
-// y[t] = sum_j wts[t, j] rows[pos[t top + j]] + gate[t] shared[t];  x[t] += y / rms(y) * w.  One workgroup per token; y stays in
-// registers between the two passes (width <= 256 x 16).
-__global__ __launch_bounds__(256) void moe_combine_norm_add_kernel(float* x, uint16_t* xcopy, const float* rows, const int32_t* pos,
-                                                                   const float* wts, const float* shared, const float* sgate, const float* w,
-                                                                   int width, int top, float eps) {
+// y[t] = sum_j wts[t, j] rows[pos[t top + j]] + gate[t] shared[t];  x[t] += y / rms(y) * w.  One workgroup per token; the token's row
+// indices and weights go through LDS first (so that the row loads do not wait on them one after the other); y stays in registers
+// between the two passes (width <= 256 x 16).  VEC: 16-byte accesses (width a multiple of 4).
+template <bool VEC> __global__ __launch_bounds__(256) void moe_combine_norm_add_kernel(float* __restrict__ x, uint16_t* __restrict__ xcopy,
+                                                                                       const float* __restrict__ rows, const int32_t* __restrict__ pos,
+                                                                                       const float* __restrict__ wts, const float* __restrict__ shared,
+                                                                                       const float* __restrict__ sgate, const float* __restrict__ w,
+                                                                                       int width, int top, float eps) {
     __shared__ float red[4];
+    extern __shared__ int csm[];
+    int* sp = csm;                                      // [top] rows of the token's pairs
+    float* sw = reinterpret_cast<float*>(csm + top);    // [top] their weights
     const int t = blockIdx.x;
+    for (int j = threadIdx.x; j < top; j += blockDim.x) { sp[j] = pos[(size_t)t * top + j]; sw[j] = wts[(size_t)t * top + j]; }
+    __syncthreads();
+    constexpr int E = VEC ? 4 : 1, U = 16 / E;
     float y[16];
     float ss = 0.f;
     const float sg = shared ? (sgate ? sgate[t] : 1.f) : 0.f;
 #pragma unroll
-    for (int u = 0; u < 16; ++u) {
-        const int i = threadIdx.x + 256 * u;
-        float a = 0.f;
+    for (int u = 0; u < U; ++u) {
+        const int i = (threadIdx.x + 256 * u) * E;
+        float a[E];
+#pragma unroll
+        for (int e = 0; e < E; ++e) a[e] = 0.f;
         if (i < width) {
-            for (int j = 0; j < top; ++j) a = fmaf(wts[(size_t)t * top + j], rows[(size_t)pos[(size_t)t * top + j] * width + i], a);
-            if (shared) a = fmaf(sg, shared[(size_t)t * width + i], a);
+            for (int j = 0; j < top; ++j) {
+                const float* r = rows + (size_t)sp[j] * width + i;
+                if (VEC) { const float4 v = *reinterpret_cast<const float4*>(r); a[0] = fmaf(sw[j], v.x, a[0]); a[E > 1 ? 1 : 0] = fmaf(sw[j], v.y, a[E > 1 ? 1 : 0]);
+                           a[E > 1 ? 2 : 0] = fmaf(sw[j], v.z, a[E > 1 ? 2 : 0]); a[E > 1 ? 3 : 0] = fmaf(sw[j], v.w, a[E > 1 ? 3 : 0]); }
+                else a[0] = fmaf(sw[j], r[0], a[0]);
+            }
+            if (shared)
+#pragma unroll
+                for (int e = 0; e < E; ++e) a[e] = fmaf(sg, shared[(size_t)t * width + i + e], a[e]);
         }
-        y[u] = a;
-        ss += a * a;
+#pragma unroll
+        for (int e = 0; e < E; ++e) { y[u * E + e] = a[e]; ss += a[e] * a[e]; }
     }
     ss = block_sum(ss, red);
     const float inv = 1.f / sqrtf(ss / (float)width + eps);
 #pragma unroll
-    for (int u = 0; u < 16; ++u) {
-        const int i = threadIdx.x + 256 * u;
-        if (i < width) {
-            const float v = x[(size_t)t * width + i] + y[u] * inv * w[i];
-            x[(size_t)t * width + i] = v;
-            if (xcopy) xcopy[(size_t)t * width + i] = f32_to_bf16(v);
+    for (int u = 0; u < U; ++u) {
+        const int i = (threadIdx.x + 256 * u) * E;
+        if (i >= width) continue;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const float v = x[(size_t)t * width + i + e] + y[u * E + e] * inv * w[i + e];
+            x[(size_t)t * width + i + e] = v;
+            if (xcopy) xcopy[(size_t)t * width + i + e] = f32_to_bf16(v);
         }
     }
 }
@@ -1914,12 +1942,13 @@ int mi355_hyb_moe_route(int32_t* expert_ids, float* weights, float* shared_gate,
     if (T <= 0) return 0;
     const size_t lds = (size_t)(width + experts + 1) * sizeof(float);
     if (lds > 60000) return -1;
-    if (xn && out_dtype == MI355_DTYPE_BF16)
-        moe_route_kernel<uint16_t><<<T, 256, lds, to_stream(stream)>>>(expert_ids, weights, shared_gate, (uint16_t*)xn, x, norm_w, router, correction,
-                                                                      gate_row, width, experts, top, scale, eps);
-    else
-        moe_route_kernel<float><<<T, 256, lds, to_stream(stream)>>>(expert_ids, weights, shared_gate, (float*)xn, x, norm_w, router, correction,
-                                                                   gate_row, width, experts, top, scale, eps);
+    // few tokens (decoding batches): sixteen waves per token, about one router row each; prompts: four
+    const bool bf = xn && out_dtype == MI355_DTYPE_BF16;
+#define ROUTE(TO, NW) moe_route_kernel<TO, NW><<<T, 64 * NW, lds, to_stream(stream)>>>(expert_ids, weights, shared_gate, (TO*)xn, x, norm_w, router, \
+                                                                                       correction, gate_row, width, experts, top, scale, eps)
+    if (T <= 256) { if (bf) ROUTE(uint16_t, 16); else ROUTE(float, 16); }
+    else { if (bf) ROUTE(uint16_t, 4); else ROUTE(float, 4); }
+#undef ROUTE
     LAUNCH_OK(); return 0;
 }
 
@@ -1990,7 +2019,12 @@ int mi355_hyb_moe_combine_norm_add(float* x, void* xcopy, const float* y_rows, c
                                    float eps, int64_t stream) {
     if (!x || !y_rows || !pos || !weights || !w || width <= 0 || width > 4096 || top < 1) return -1;
     if (T <= 0) return 0;
-    moe_combine_norm_add_kernel<<<T, 256, 0, to_stream(stream)>>>(x, (uint16_t*)xcopy, y_rows, pos, weights, y_shared, shared_gate, w, width, top, eps);
+    const size_t lds = (size_t)top * 8;
+    if (top > 4096) return -1;
+    if (width % 4 == 0 && (uintptr_t)y_rows % 16 == 0)
+        moe_combine_norm_add_kernel<true><<<T, 256, lds, to_stream(stream)>>>(x, (uint16_t*)xcopy, y_rows, pos, weights, y_shared, shared_gate, w, width, top, eps);
+    else
+        moe_combine_norm_add_kernel<false><<<T, 256, lds, to_stream(stream)>>>(x, (uint16_t*)xcopy, y_rows, pos, weights, y_shared, shared_gate, w, width, top, eps);
     LAUNCH_OK(); return 0;
 }
 
