@@ -896,6 +896,173 @@ void window_attention_mfma_kernel(AttnArgs p) {
     }
 }
 
+// The same prompt-sized step for grouped-query attention: a workgroup of HPG waves takes HPG query heads that share ONE key/value head
+// for the same tile of 16 tokens -- same keys, same mask -- so the 64 key rows and the transposed 64 value rows of a chunk are staged in
+// LDS once per workgroup (cooperatively, the next chunk's rows already in flight in registers) instead of once per head from L2, and
+// the key fragments of S = Q K^T are 16-byte LDS reads.  Softmax, the two probability planes and the products are as above, per wave.
+template <int DK, int VT, int HPG> __global__ __launch_bounds__(64 * HPG) void window_attention_group_kernel(AttnArgs p) {
+    constexpr int RS = 72;                                           // bf16 per row of P and V^T: 64 keys + 8 of padding
+    constexpr int KRS = DK * 32 + 8;                                 // bf16 per staged key row (16 rows of a fragment read: 16 different bank groups)
+    constexpr int NT = 64 * HPG;
+    constexpr int KCH = DK * 4;                                      // 16-byte chunks of a key row
+    constexpr int KPT = KCH / HPG > 0 ? KCH / HPG : 1;               // key chunks per thread and stage (HPG divides 4 DK)
+    constexpr int VPT = (VT * 2 + HPG - 1) / HPG;                    // value chunks (8 columns) per wave and stage
+    static_assert(KCH % HPG == 0, "4 DK must be a multiple of HPG");
+    __shared__ __align__(16) uint16_t Ks[64 * KRS], Vt[VT * 16 * RS], Ph[HPG][16 * RS], Pl[HPG][16 * RS];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, m16 = lane & 15, kg = lane >> 4;
+    int b = blockIdx.x, s = 0, n_new = 0;
+    for (; s < p.n_seqs; ++s) {
+        n_new = (int)(p.cu_q[s + 1] - p.cu_q[s]);
+        const int tiles = (n_new + 15) >> 4;
+        if (b < tiles) break;
+        b -= tiles;
+    }
+    if (s >= p.n_seqs) return;
+    const int t0 = (int)p.cu_q[s] + b * 16, nq = min(16, (int)p.cu_q[s + 1] - t0);
+    const int pos0 = (int)p.ctx[s] - n_new + b * 16;
+    const int h = blockIdx.y * HPG + wave, g = h / (p.H / p.G), d = p.d, vd = p.vd;
+    const uint16_t* Q = static_cast<const uint16_t*>(p.q);
+    const uint16_t* K = static_cast<const uint16_t*>(p.k_pages);
+    const uint16_t* V = static_cast<const uint16_t*>(p.v_pages);
+    const uint32_t* bt = p.bt + (size_t)s * p.max_blocks;
+    uint4 qf[DK];
+#pragma unroll
+    for (int ks = 0; ks < DK; ++ks)
+        qf[ks] = m16 < nq ? *reinterpret_cast<const uint4*>(Q + ((size_t)(t0 + m16) * p.H + h) * d + ks * 32 + 8 * kg) : uint4{0, 0, 0, 0};
+    float mrow[4], lrow[4];
+    f32x4_t acc[VT];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) { mrow[v] = -INFINITY; lrow[v] = 0.f; }
+#pragma unroll
+    for (int c = 0; c < VT; ++c) acc[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    const int hi = pos0 + nq - 1;
+    const int lo = p.window > 0 ? max(0, pos0 - p.window + 1) : 0;
+    const int nkeep = min(p.keep, lo), n_vis = nkeep + hi - lo + 1;
+    auto key_at = [&](int i) { return i < nkeep ? i : (i < n_vis ? lo + (i - nkeep) : hi + 1); };
+    auto page_row = [&](int key) { return (size_t)bt[key / p.bs] * p.bs + (key % p.bs); };
+    uint4 kreg[KPT], vreg[VPT];
+    auto fetch = [&](int j0) {
+#pragma unroll
+        for (int n = 0; n < KPT; ++n) {
+            const int idx = tid + n * NT, ki = idx / KCH, c = idx - ki * KCH;
+            const int key = key_at(j0 + ki);
+            kreg[n] = key <= hi ? *reinterpret_cast<const uint4*>(K + page_row(key) * p.k_ld + g * d + c * 8) : uint4{0, 0, 0, 0};
+        }
+        const int vkey = key_at(j0 + lane);
+        const uint16_t* vrow = V + (vkey <= hi ? page_row(vkey) : 0) * p.v_ld + g * vd;
+#pragma unroll
+        for (int n = 0; n < VPT; ++n) {
+            const int c8 = wave + n * HPG;
+            vreg[n] = (vkey <= hi && c8 < VT * 2) ? *reinterpret_cast<const uint4*>(vrow + c8 * 8) : uint4{0, 0, 0, 0};
+        }
+    };
+    auto stage = [&]() {
+#pragma unroll
+        for (int n = 0; n < KPT; ++n) {
+            const int idx = tid + n * NT, ki = idx / KCH, c = idx - ki * KCH;
+            *reinterpret_cast<uint4*>(&Ks[ki * KRS + c * 8]) = kreg[n];
+        }
+        // transposing store of the value rows (zeros past the end): the lane pair (2a, 2a + 1) swaps words, every lane writes one 4-byte
+        // word = two keys of one column
+        const int col_odd = lane & 1, key_even = lane & ~1;
+#pragma unroll
+        for (int n = 0; n < VPT; ++n) {
+            const int c8 = wave + n * HPG;
+            if (c8 >= VT * 2) break;
+            const uint32_t w[4] = {vreg[n].x, vreg[n].y, vreg[n].z, vreg[n].w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t other = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)w[e], 0xB1, 0xF, 0xF, true);   // quad_perm [1, 0, 3, 2]
+                const uint32_t pair = col_odd ? ((other >> 16) | (w[e] & 0xFFFF0000u)) : ((w[e] & 0xFFFFu) | (other << 16));
+                *reinterpret_cast<uint32_t*>(&Vt[(c8 * 8 + 2 * e + col_odd) * RS + key_even]) = pair;
+            }
+        }
+    };
+    uint16_t* ph = Ph[wave];
+    uint16_t* pl = Pl[wave];
+    fetch(0);
+    for (int j0 = 0; j0 < n_vis; j0 += 64) {
+        __syncthreads();                                             // the chunk before is multiplied: its rows may go
+        stage();
+        __syncthreads();
+        if (j0 + 64 < n_vis) fetch(j0 + 64);
+        f32x4_t sacc[4];
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) {
+            sacc[kt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int ks = 0; ks < DK; ++ks) {
+                const uint4 kf = *reinterpret_cast<const uint4*>(&Ks[(kt * 16 + m16) * KRS + ks * 32 + 8 * kg]);
+                sacc[kt] = mfma_bf16(qf[ks], kf, sacc[kt]);
+            }
+        }
+        float mx[4], sc[4][4];
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const int r = 4 * kg + v, qpos = pos0 + r;
+            mx[v] = -INFINITY;
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt) {
+                const int key = key_at(j0 + kt * 16 + m16);
+                const bool ok_ = r < nq && key <= qpos && (p.window == 0 || qpos - key < p.window || key < p.keep);
+                sc[v][kt] = ok_ ? cap_score(sacc[kt][v] * p.scale, p.softcap) : -INFINITY;
+                mx[v] = fmaxf(mx[v], sc[v][kt]);
+            }
+#pragma unroll
+            for (int o = 1; o < 16; o <<= 1) mx[v] = fmaxf(mx[v], __shfl_xor(mx[v], o));
+        }
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const float mn = fmaxf(mrow[v], mx[v]);
+            const float corr = (mn == -INFINITY || mrow[v] == -INFINITY) ? (mn == -INFINITY ? 1.f : 0.f) : expf(mrow[v] - mn);
+            float rs = 0.f;
+#pragma unroll
+            for (int kt = 0; kt < 4; ++kt) {
+                const float pv = sc[v][kt] == -INFINITY ? 0.f : expf(sc[v][kt] - mn);
+                rs += pv;
+                const uint16_t hb = f32_to_bf16(pv);
+                ph[(4 * kg + v) * RS + kt * 16 + m16] = hb;
+                pl[(4 * kg + v) * RS + kt * 16 + m16] = f32_to_bf16(pv - bf16_to_f32(hb));
+            }
+#pragma unroll
+            for (int o = 1; o < 16; o <<= 1) rs += __shfl_xor(rs, o);
+            lrow[v] = lrow[v] * corr + rs;
+            mrow[v] = mn;
+#pragma unroll
+            for (int c = 0; c < VT; ++c) acc[c][v] *= corr;
+        }
+        __syncthreads();                                             // this wave's probability planes are written
+#pragma unroll
+        for (int k2 = 0; k2 < 2; ++k2) {
+            const uint4 ah = *reinterpret_cast<const uint4*>(&ph[m16 * RS + k2 * 32 + 8 * kg]);
+            const uint4 al = *reinterpret_cast<const uint4*>(&pl[m16 * RS + k2 * 32 + 8 * kg]);
+#pragma unroll
+            for (int c = 0; c < VT; ++c) {
+                const uint4 vf = *reinterpret_cast<const uint4*>(&Vt[(c * 16 + m16) * RS + k2 * 32 + 8 * kg]);
+                acc[c] = mfma_bf16(ah, vf, acc[c]);
+                acc[c] = mfma_bf16(al, vf, acc[c]);
+            }
+        }
+    }
+    const float sink = p.sink ? p.sink[h] : -INFINITY;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        const int r = 4 * kg + v;
+        if (r >= nq) continue;
+        const float M = fmaxf(mrow[v], sink);
+        const float cm = expf(mrow[v] - M);
+        const float L = lrow[v] * cm + (p.sink ? expf(sink - M) : 0.f);
+        const float f = cm / L * p.out_scale;
+        const size_t base = (size_t)(t0 + r) * p.ldo + p.out_off + (size_t)h * vd;
+#pragma unroll
+        for (int c = 0; c < VT; ++c) {
+            const float o = acc[c][v] * f;
+            if (p.out_f32) static_cast<float*>(p.out)[base + c * 16 + m16] = o;
+            else static_cast<uint16_t*>(p.out)[base + c * 16 + m16] = f32_to_bf16(o);
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------------------------------ short convolution
 struct ConvArgs {
     float* out; const float* proj; int ldp, off; const float* w; float* state; int64_t state_stride;
@@ -1498,6 +1665,7 @@ __global__ void scale_f32_kernel(float* x, float s, int64_t n) {
     if (i < n) x[i] *= s;
 }
 
+int g_attn_group = 1;           // 0: grouped-query prompt steps take the kernel with one wave per head (A/B, tests of both paths)
 int g_attn_mfma = 1;            // mi355_hyb_set_attention_mfma(0): prompt steps take the generic kernel too (A/B, tests of both paths)
 
 #define LAUNCH_OK() do { const hipError_t e_ = hipGetLastError(); if (e_ != hipSuccess) return (int)e_; } while (0)
@@ -1513,7 +1681,7 @@ int mi355_hyb_token_seq(int32_t* tok_seq, const uint32_t* cu_seqlens_q, int32_t 
     token_seq_kernel<<<num_seqs, 64, 0, to_stream(stream)>>>(tok_seq, cu_seqlens_q, num_seqs);
     LAUNCH_OK(); return 0;
 }
-void mi355_hyb_set_attention_mfma(int32_t on) { g_attn_mfma = on ? 1 : 0; }
+void mi355_hyb_set_attention_mfma(int32_t on) { g_attn_mfma = on ? 1 : 0; g_attn_group = on == 2 ? 0 : 1; }
 int mi355_hyb_bf16_to_f32(float* out, const uint16_t* in, int64_t n, int64_t stream) {
     if (n <= 0) return 0;
     bf16_to_f32_kernel<<<(unsigned)((n + 255) / 256), 256, 0, to_stream(stream)>>>(out, in, n);
@@ -1688,6 +1856,18 @@ int mi355_hyb_masked_attention(void* out, int32_t out_dtype, int32_t ldo, int32_
     if (!f && T >= 64 && dim % 32 == 0 && dim <= 256 && vdim % 16 == 0 && vdim <= 256 && (uintptr_t)q % 16 == 0 && (uintptr_t)k_pages % 16 == 0 &&
         (uintptr_t)v_pages % 16 == 0 && k_ld % 8 == 0 && v_ld % 8 == 0 && g_attn_mfma) {
         const int dk = dim / 32, vt = vdim / 16;
+        // grouped-query attention: the query heads of a key/value head share a workgroup and its staged rows
+        const int hpg = cross ? 1 : ((heads / kv_heads) % 4 == 0 ? 4 : (heads / kv_heads) % 2 == 0 ? 2 : 1);
+        if (hpg > 1 && dk <= 4 && vt <= 8 && vt % 2 == 0 && g_attn_group) {
+            const dim3 ggrid((T + 15) / 16 + num_seqs, heads / hpg, 1);
+#define WG2(DK, VT) do { if (hpg == 4) window_attention_group_kernel<DK, VT, 4><<<ggrid, 256, 0, s_>>>(p); \
+                         else window_attention_group_kernel<DK, VT, 2><<<ggrid, 128, 0, s_>>>(p); } while (0)
+#define WGV(DK) do { switch (vt) { case 2: WG2(DK, 2); break; case 4: WG2(DK, 4); break; case 6: WG2(DK, 6); break; default: WG2(DK, 8); break; } } while (0)
+            switch (dk) { case 1: WGV(1); break; case 2: WGV(2); break; case 3: WGV(3); break; default: WGV(4); break; }
+#undef WGV
+#undef WG2
+            LAUNCH_OK(); return 0;
+        }
         // cross mode: 2 value heads per block where the head sizes have such a build (dim <= 128, vdim <= 128), the rest of the
         // key/value heads along z (4 per block: one wave per SIMD, measured 1.4 x slower)
         const int nv = (cross && dk <= 4 && vt <= 8) ? (kv_heads % 2 == 0 ? 2 : 1) : 1;

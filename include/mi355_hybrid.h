@@ -313,7 +313,8 @@ int mi355_hyb_moe_combine_norm_add(float* x, void* xcopy, const float* y_rows, c
                                    const float* y_shared, const float* shared_gate, const float* w, int32_t num_tokens, int32_t width,
                                    int32_t top, float eps, int64_t stream);
 int mi355_hyb_scale_f32(float* x, float s, int64_t n, int64_t stream);
-/* 0: prompt-sized steps over bf16 pages take the generic kernel instead of the matrix-core one (A/B switch, process-wide; default 1) */
+/* 0: prompt-sized steps over bf16 pages take the generic kernel instead of the matrix-core ones; 2: the matrix-core kernel with one
+ * wave per head also where the query heads of a key/value head could share a workgroup (A/B switch, process-wide; default 1) */
 void mi355_hyb_set_attention_mfma(int32_t on);
 /* short causal convolution over time per channel, then silu: out f32 [T, channels] from proj columns [off, off + channels);
  * the taps - 1 inputs before a portion come from conv_state f32 [slots, channels, taps - 1] (zeros at position 0);

@@ -208,7 +208,7 @@ def test_window_that_keeps_the_first_tokens(lib, dtype, Hh, G, d, vd, window, ke
     ok(lib.mi355_hyb_token_seq(seq.data_ptr(), P(cu, np.uint32), 2, _st()))
     dq, dk_, dv_ = dev_dt(np.concatenate(qs), dtype), dev_dt(kp, dtype), dev_dt(vp, dtype)
     wantc = np.concatenate(want)
-    for mfma in (1, 0):
+    for mfma in (1, 2, 0):              # heads of a group in one workgroup; a wave per head; the generic kernel
         lib.mi355_hyb_set_attention_mfma(mfma)
         out = torch.zeros((T, Hh * vd), device="cuda")
         ok(lib.mi355_hyb_masked_attention(out.data_ptr(), F32, Hh * vd, 0, dq.data_ptr(), dk_.data_ptr(), dv_.data_ptr(), P(bt, np.uint32),
