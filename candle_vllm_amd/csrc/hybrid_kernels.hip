@@ -905,9 +905,8 @@ template <int DK, int VT, int HPG> __global__ __launch_bounds__(64 * HPG) void w
     constexpr int KRS = DK * 32 + 8;                                 // bf16 per staged key row (16 rows of a fragment read: 16 different bank groups)
     constexpr int NT = 64 * HPG;
     constexpr int KCH = DK * 4;                                      // 16-byte chunks of a key row
-    constexpr int KPT = KCH / HPG > 0 ? KCH / HPG : 1;               // key chunks per thread and stage (HPG divides 4 DK)
+    constexpr int KPT = (64 * KCH + NT - 1) / NT;                    // key chunks per thread and stage
     constexpr int VPT = (VT * 2 + HPG - 1) / HPG;                    // value chunks (8 columns) per wave and stage
-    static_assert(KCH % HPG == 0, "4 DK must be a multiple of HPG");
     __shared__ __align__(16) uint16_t Ks[64 * KRS], Vt[VT * 16 * RS], Ph[HPG][16 * RS], Pl[HPG][16 * RS];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, m16 = lane & 15, kg = lane >> 4;
     int b = blockIdx.x, s = 0, n_new = 0;
@@ -945,7 +944,7 @@ template <int DK, int VT, int HPG> __global__ __launch_bounds__(64 * HPG) void w
 #pragma unroll
         for (int n = 0; n < KPT; ++n) {
             const int idx = tid + n * NT, ki = idx / KCH, c = idx - ki * KCH;
-            const int key = key_at(j0 + ki);
+            const int key = ki < 64 ? key_at(j0 + ki) : hi + 1;
             kreg[n] = key <= hi ? *reinterpret_cast<const uint4*>(K + page_row(key) * p.k_ld + g * d + c * 8) : uint4{0, 0, 0, 0};
         }
         const int vkey = key_at(j0 + lane);
@@ -960,7 +959,7 @@ template <int DK, int VT, int HPG> __global__ __launch_bounds__(64 * HPG) void w
 #pragma unroll
         for (int n = 0; n < KPT; ++n) {
             const int idx = tid + n * NT, ki = idx / KCH, c = idx - ki * KCH;
-            *reinterpret_cast<uint4*>(&Ks[ki * KRS + c * 8]) = kreg[n];
+            if (ki < 64) *reinterpret_cast<uint4*>(&Ks[ki * KRS + c * 8]) = kreg[n];
         }
         // transposing store of the value rows (zeros past the end): the lane pair (2a, 2a + 1) swaps words, every lane writes one 4-byte
         // word = two keys of one column
@@ -1857,10 +1856,11 @@ int mi355_hyb_masked_attention(void* out, int32_t out_dtype, int32_t ldo, int32_
         (uintptr_t)v_pages % 16 == 0 && k_ld % 8 == 0 && v_ld % 8 == 0 && g_attn_mfma) {
         const int dk = dim / 32, vt = vdim / 16;
         // grouped-query attention: the query heads of a key/value head share a workgroup and its staged rows
-        const int hpg = cross ? 1 : ((heads / kv_heads) % 4 == 0 ? 4 : (heads / kv_heads) % 2 == 0 ? 2 : 1);
+        const int hpk = heads / kv_heads, hpg = cross ? 1 : (hpk % 4 == 0 ? 4 : hpk % 3 == 0 ? 3 : hpk % 2 == 0 ? 2 : 1);
         if (hpg > 1 && dk <= 4 && vt <= 8 && vt % 2 == 0 && g_attn_group) {
             const dim3 ggrid((T + 15) / 16 + num_seqs, heads / hpg, 1);
 #define WG2(DK, VT) do { if (hpg == 4) window_attention_group_kernel<DK, VT, 4><<<ggrid, 256, 0, s_>>>(p); \
+                         else if (hpg == 3) window_attention_group_kernel<DK, VT, 3><<<ggrid, 192, 0, s_>>>(p); \
                          else window_attention_group_kernel<DK, VT, 2><<<ggrid, 128, 0, s_>>>(p); } while (0)
 #define WGV(DK) do { switch (vt) { case 2: WG2(DK, 2); break; case 4: WG2(DK, 4); break; case 6: WG2(DK, 6); break; default: WG2(DK, 8); break; } } while (0)
             switch (dk) { case 1: WGV(1); break; case 2: WGV(2); break; case 3: WGV(3); break; default: WGV(4); break; }

@@ -169,7 +169,8 @@ def _scatter(n_rows, bs, free):
 @pytest.mark.parametrize("Hh,G,d,vd,window,keep,bs,big", [(4, 2, 24, 40, 20, 5, 16, False), (3, 3, 8, 8, 9, 0, 8, False), (2, 1, 16, 130, 7, 30, 32, False),
                                                           (1, 1, 4, 2, 1, 1, 4, False), (2, 2, 16, 16, 0, 6, 16, False),
                                                           # prompt-sized steps; bf16 pages take the matrix-core kernel
-                                                          (4, 2, 64, 48, 50, 11, 16, True), (6, 1, 96, 64, 80, 24, 64, True), (2, 1, 32, 16, 100, 130, 64, True)])
+                                                          (4, 2, 64, 48, 50, 11, 16, True), (6, 1, 96, 64, 80, 24, 64, True), (2, 1, 32, 16, 100, 130, 64, True),
+                                                          (6, 2, 32, 32, 40, 7, 16, True), (3, 1, 128, 128, 0, 0, 32, True), (5, 1, 64, 64, 30, 2, 16, True)])
 def test_window_that_keeps_the_first_tokens(lib, dtype, Hh, G, d, vd, window, keep, bs, big):
     """two unequal sequences in shuffled pages.  Dominant keys sit at the last kept position and at the first one that is not kept, at
     the window's first position and just below it -- seen from a late query each of them decides the output or must not be seen at all"""
