@@ -409,7 +409,7 @@ _sig("mi355_hyb_conv_residual", ctypes.c_int, [c_vp, c_i32, c_vp, c_i32, c_i32, 
 _sig("mi355_hyb_attn_prepare_ex", ctypes.c_int, [c_vp] * 4 + [c_i32] * 4 + [c_vp] * 6 + [c_i32] * 8 + [c_vp, c_f32, c_i32, c_i64])
 _sig("mi355_hyb_masked_attention", ctypes.c_int, [c_vp, c_i32, c_i32, c_i32] + [c_vp] * 8 + [c_i32] * 10 + [c_f32, c_f32, c_i32, c_i32, c_f32,
                                                                                                       c_i32, c_i32, c_i64])
-_sig("mi355_hyb_moe_route", ctypes.c_int, [c_vp, c_vp, c_vp, c_vp, c_i32, c_vp, c_vp, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_f32, c_f32, c_i64])
+_sig("mi355_hyb_moe_route", ctypes.c_int, [c_vp, c_vp, c_vp, c_vp, c_i32, c_vp, c_vp, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_f32, c_f32, c_i32, c_i64])
 _sig("mi355_hyb_moe_block_rows", c_i32, [c_i32] * 5)
 _sig("mi355_hyb_moe_group", ctypes.c_int, [c_vp, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_i64])
 _sig("mi355_hyb_linear_grouped", ctypes.c_int, [c_vp, c_i32, c_vp, c_i32, c_i32, c_vp, c_vp, c_i64, c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_i64])

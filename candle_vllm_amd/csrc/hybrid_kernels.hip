@@ -1490,7 +1490,7 @@ template <typename TO> __global__ void head_gate_kernel(TO* out, const float* in
 template <typename TO, int NW> __global__ __launch_bounds__(64 * NW) void moe_route_kernel(int32_t* ids, float* wts, float* sgate, TO* xn, const float* x,
                                                                                const float* norm_w, const float* router, const float* corr,
                                                                                const float* gate_row, int width, int E, int K, float scale,
-                                                                               float eps) {
+                                                                               float eps, int append) {
     extern __shared__ __align__(16) float rsm[];
     float* hs = rsm;                       // [width]
     float* logit = hs + width;             // [E + 1]
@@ -1534,7 +1534,12 @@ template <typename TO, int NW> __global__ __launch_bounds__(64 * NW) void moe_ro
     }
     __syncthreads();
     if (wave != 0) return;
-    if (gate_row && lane == 0) sgate[t] = sigmoidf_(logit[E]);
+    const int KS = K + (append ? 1 : 0);                                // pairs per token: the shared expert as one more pair of every token
+    if (gate_row && lane == 0) {
+        const float sg = sigmoidf_(logit[E]);
+        if (sgate) sgate[t] = sg;
+        if (append) { ids[(size_t)t * KS + K] = E; wts[(size_t)t * KS + K] = sg; }
+    }
     float m = -INFINITY;
     for (int e = lane; e < E; e += 64) m = fmaxf(m, logit[e]);
     m = wave_max(m);
@@ -1555,8 +1560,8 @@ template <typename TO, int NW> __global__ __launch_bounds__(64 * NW) void moe_ro
         for (int o = 32; o > 0; o >>= 1) cand = min(cand, __shfl_xor(cand, o));
         if (lane == (cand & 63)) taken |= 1ull << (cand >> 6);
         if (lane == 0) {
-            ids[(size_t)t * K + j] = cand;
-            wts[(size_t)t * K + j] = expf(logit[cand] - m) / den * scale;
+            ids[(size_t)t * KS + j] = cand;
+            wts[(size_t)t * KS + j] = expf(logit[cand] - m) / den * scale;
         }
     }
 }
@@ -2116,16 +2121,16 @@ int mi355_hyb_scale_f32(float* x, float s, int64_t n, int64_t stream) {
 
 int mi355_hyb_moe_route(int32_t* expert_ids, float* weights, float* shared_gate, void* xn, int32_t out_dtype, const float* x,
                         const float* norm_w, const float* router, const float* correction, const float* gate_row, int32_t T,
-                        int32_t width, int32_t experts, int32_t top, float scale, float eps, int64_t stream) {
+                        int32_t width, int32_t experts, int32_t top, float scale, float eps, int32_t append_shared, int64_t stream) {
     if (!expert_ids || !weights || !x || !router || width <= 0 || experts < 1 || experts > 4096 || top < 1 || top > experts) return -1;
-    if ((gate_row && !shared_gate) || (xn && !is_dt(out_dtype))) return -1;
+    if ((gate_row && !shared_gate && !append_shared) || (append_shared && !gate_row) || (xn && !is_dt(out_dtype))) return -1;
     if (T <= 0) return 0;
     const size_t lds = (size_t)(width + experts + 1) * sizeof(float);
     if (lds > 60000) return -1;
     // few tokens (decoding batches): sixteen waves per token, about one router row each; prompts: four
     const bool bf = xn && out_dtype == MI355_DTYPE_BF16;
 #define ROUTE(TO, NW) moe_route_kernel<TO, NW><<<T, 64 * NW, lds, to_stream(stream)>>>(expert_ids, weights, shared_gate, (TO*)xn, x, norm_w, router, \
-                                                                                       correction, gate_row, width, experts, top, scale, eps)
+                                                                                       correction, gate_row, width, experts, top, scale, eps, append_shared ? 1 : 0)
     if (T <= 256) { if (bf) ROUTE(uint16_t, 16); else ROUTE(float, 16); }
     else { if (bf) ROUTE(uint16_t, 4); else ROUTE(float, 4); }
 #undef ROUTE

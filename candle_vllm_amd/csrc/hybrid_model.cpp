@@ -59,6 +59,8 @@ struct HLayer {
     int conv_channels() const { return 2 * c.d_kv_heads * c.d_dim + c.d_heads * c.d_vdim; }
     int a_conv_channels() const { return (c.a_heads + c.a_kv_heads) * c.a_dim + c.a_kv_heads * c.a_vdim; }
     // elements of a token's row in the key / value pages (latent attention: one row [latent | rotated key part], no value pages)
+    // a shared expert of the experts' size runs as one more group of the grouped products (and one more pair of every token)
+    bool shared_merged() const { return c.mlp_kind == 3 && c.moe_shared_ff > 0 && c.moe_shared_ff == c.mlp_ff; }
     int k_row() const { return is_latent() ? c.a_kv_rank + c.a_rot_dim : c.a_kv_heads * c.a_dim; }
     int v_row() const { return is_latent() ? 0 : c.a_kv_heads * c.a_vdim; }
 };
@@ -196,8 +198,8 @@ int64_t expected_elems(const HModel* m, int layer, int which) {
         case MI355_HW_IN_CONV: return c.in_conv ? (int64_t)W * c.in_conv : -1;
         case MI355_HW_MOE_ROUTER: return c.mlp_kind == 3 ? (int64_t)(c.moe_experts + (c.moe_shared_ff ? 1 : 0)) * W : -1;
         case MI355_HW_MOE_CORRECTION: return c.mlp_kind == 3 ? c.moe_experts : -1;
-        case MI355_HW_MOE_GATE_UP: return c.mlp_kind == 3 ? (int64_t)c.moe_experts * 2 * c.mlp_ff * W : -1;
-        case MI355_HW_MOE_DOWN: return c.mlp_kind == 3 ? (int64_t)c.moe_experts * W * c.mlp_ff : -1;
+        case MI355_HW_MOE_GATE_UP: return c.mlp_kind == 3 ? (int64_t)(c.moe_experts + L.shared_merged()) * 2 * c.mlp_ff * W : -1;
+        case MI355_HW_MOE_DOWN: return c.mlp_kind == 3 ? (int64_t)(c.moe_experts + L.shared_merged()) * W * c.mlp_ff : -1;
         case MI355_HW_A_SINK: return (L.has_attn() || L.is_latent()) && c.a_has_sink ? c.a_heads : -1;
         case MI355_HW_A_CONV: return L.is_conv_attn() ? (int64_t)L.a_conv_channels() * c.a_conv : -1;
         case MI355_HW_A_TALK: return L.is_conv_attn() && c.a_talk ? c.a_heads * c.a_heads : -1;
@@ -210,9 +212,9 @@ int64_t expected_elems(const HModel* m, int layer, int which) {
         case MI355_HW_D_NORM: return L.has_delta() ? c.d_vdim : -1;
         case MI355_HW_D_A2: return L.has_delta() && c.d_decay_channels ? (int64_t)c.d_heads * c.d_dim * c.d_a_rank : -1;
         case MI355_HW_D_G2: return L.has_delta() && c.d_gate == MI355_HYB_GATE_SIGMOID_LR ? (int64_t)c.d_heads * c.d_vdim * c.d_g_rank : -1;
-        case MI355_HW_MLP_GATE_UP: if (c.mlp_kind == 3) return c.moe_shared_ff ? (int64_t)2 * c.moe_shared_ff * W : -1;
+        case MI355_HW_MLP_GATE_UP: if (c.mlp_kind == 3) return c.moe_shared_ff && !L.shared_merged() ? (int64_t)2 * c.moe_shared_ff * W : -1;
                                    return c.mlp_kind ? (int64_t)2 * c.mlp_ff * W : -1;
-        case MI355_HW_MLP_DOWN: if (c.mlp_kind == 3) return c.moe_shared_ff ? (int64_t)W * c.moe_shared_ff : -1;
+        case MI355_HW_MLP_DOWN: if (c.mlp_kind == 3) return c.moe_shared_ff && !L.shared_merged() ? (int64_t)W * c.moe_shared_ff : -1;
                                 return c.mlp_kind ? (int64_t)W * c.mlp_ff : -1;
         default: return -1;
     }
@@ -360,8 +362,8 @@ void* mi355_hybrid_create(const mi355_hybrid_config* cfg, const mi355_hybrid_lay
         if (c.mixer == MI355_HYB_MIX_MINGRU) { L.state_off = off; off += c.g_width; }
         if (c.in_conv) { L.in_conv_off = off; off += (int64_t)cfg->width * (c.in_conv - 1); m->need_pre = true; }
         if (c.mlp_kind == 3) {
-            m->max_moe_experts = std::max(m->max_moe_experts, c.moe_experts);
-            m->max_moe_top = std::max(m->max_moe_top, c.moe_top);
+            m->max_moe_experts = std::max(m->max_moe_experts, c.moe_experts + 1);
+            m->max_moe_top = std::max(m->max_moe_top, c.moe_top + 1);
             m->max_moe_ff = std::max(m->max_moe_ff, c.mlp_ff);
             m->max_ff = std::max(m->max_ff, c.moe_shared_ff);
         } else if (c.mlp_kind) m->max_ff = std::max(m->max_ff, c.mlp_ff);
@@ -606,13 +608,16 @@ static int forward_enqueue(HModel* m, const uint32_t* tokens, const int64_t* pos
         HCHECK(residual(MI355_HW_NORM1));
         if (c.mlp_kind == 3) {
             // mixture of experts: route (with the norm in front of it in form 2), group the (token, expert) pairs into whole blocks per
-            // expert, one grouped product for all gate/up matrices, silu, one for all down matrices; the shared expert as dense
-            // products; the weighted sum, the shared expert's gate and the output norm in one launch
-            const int E = c.moe_experts, K = c.moe_top, ff = c.mlp_ff, fs = c.moe_shared_ff, pairs = T * K;
+            // expert, one grouped product for all gate/up matrices, silu, one for all down matrices; the shared expert as one more
+            // group of every token (when it has the experts' size) or as dense products; the weighted sum, the shared expert's gate and
+            // the output norm in one launch
+            const bool merged = L.shared_merged();
+            const int E = c.moe_experts + merged, K = c.moe_top + merged, ff = c.mlp_ff, fs = merged ? 0 : c.moe_shared_ff, pairs = T * K;
             const float* router = f(MI355_HW_MOE_ROUTER);
             HCHECK(mi355_hyb_moe_route(m->moe_ids, m->moe_wts, m->moe_sgate, sandwich ? m->pre : nullptr, dt, m->x,
                                        sandwich ? f(MI355_HW_PRE_NORM2) : nullptr, router, f(MI355_HW_MOE_CORRECTION),
-                                       fs ? router + (size_t)E * W : nullptr, T, W, E, K, c.moe_scale, eps, stream));
+                                       c.moe_shared_ff ? router + (size_t)c.moe_experts * W : nullptr, T, W, c.moe_experts, c.moe_top, c.moe_scale,
+                                       eps, merged, stream));
             const int bm = std::min(mi355_hyb_moe_block_rows(pairs, E, 2 * ff, W, dt), mi355_hyb_moe_block_rows(pairs, E, W, ff, dt));
             const int nb = (pairs + bm - 1) / bm + E;
             HCHECK(mi355_hyb_moe_group(m->moe_pos, m->moe_row_token, m->moe_table, m->moe_ids, pairs, K, E, bm, nb, stream));

@@ -328,7 +328,10 @@ class KerolornSpec:
                 slots[HW_MOE_CORRECTION] = [m + "correction"]
             slots[HW_MOE_GATE_UP] = [m + "e%d.%s" % (e, n) for e in range(L.moe_experts) for n in ("gate", "up")]
             slots[HW_MOE_DOWN] = [m + "e%d.down" % e for e in range(L.moe_experts)]
-            if shared:
+            if shared and L.moe_shared_ff == L.mlp_ff:      # of the experts' size: one more matrix of the grouped products
+                slots[HW_MOE_GATE_UP] += [m + "shared.gate", m + "shared.up"]
+                slots[HW_MOE_DOWN] += [m + "shared.down"]
+            elif shared:
                 slots[HW_MLP_GATE_UP], slots[HW_MLP_DOWN] = [m + "shared.gate", m + "shared.up"], [m + "shared.down"]
         return L, slots, rope
 

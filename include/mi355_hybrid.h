@@ -135,7 +135,9 @@ typedef struct mi355_hybrid_config {
 #define MI355_HW_A_TEMP 27         /* [heads]                                                                        */
 #define MI355_HW_MOE_ROUTER 28     /* f32 [experts (+ 1 when moe_shared_ff: the shared expert's gate row last), width] */
 #define MI355_HW_MOE_CORRECTION 29 /* [experts] added to the softmax values for the choice only                      */
-#define MI355_HW_MOE_GATE_UP 30    /* [experts, 2 ff, width]: per expert gate rows, then up rows                     */
+#define MI355_HW_MOE_GATE_UP 30    /* [experts, 2 ff, width]: per expert gate rows, then up rows; a shared expert of the
+                                      experts' size (moe_shared_ff == mlp_ff) is one more matrix at the end, here and in
+                                      MOE_DOWN, and the dense slots stay empty                                       */
 #define MI355_HW_MOE_DOWN 31       /* [experts, width, ff]                                                           */
 #define MI355_HW_COUNT 32
 
@@ -286,10 +288,12 @@ int mi355_hyb_masked_attention(void* out, int32_t out_dtype, int32_t ldo, int32_
 /* mixture of experts, routing: h = RMS norm of x times norm_w (norm_w NULL: h = x) -> xn (dt_out) [T, width] (NULL = not written);
  * z = router f32 [experts, width] . h in f32, s = softmax(z); the `top` experts with the largest s + correction (correction NULL =
  * none; ties to the lower expert) -> expert_ids i32 [T, top] in descending order of the choice score, weights f32 [T, top] =
- * s[chosen] * scale.  gate_row f32 [width] or NULL: shared_gate f32 [T] = sigmoid(gate_row . h) */
+ * s[chosen] * scale.  gate_row f32 [width] or NULL: shared_gate f32 [T] (NULL = not written) = sigmoid(gate_row . h).
+ * append_shared: expert_ids and weights are [T, top + 1] and every token's last pair is (expert `experts`, that sigmoid): a shared
+ * expert of the experts' size runs as one more group of the grouped products */
 int mi355_hyb_moe_route(int32_t* expert_ids, float* weights, float* shared_gate, void* xn, int32_t out_dtype, const float* x,
                         const float* norm_w, const float* router, const float* correction, const float* gate_row, int32_t num_tokens,
-                        int32_t width, int32_t experts, int32_t top, float scale, float eps, int64_t stream);
+                        int32_t width, int32_t experts, int32_t top, float scale, float eps, int32_t append_shared, int64_t stream);
 /* rows of a grouped product's blocks that suit `pairs` (token, expert) pairs over `experts` experts with [n, k] matrices: 16 (few
  * rows per expert: a stream over the weights), 64 or 128 (matrix-core tiles through LDS) */
 int32_t mi355_hyb_moe_block_rows(int32_t pairs, int32_t experts, int32_t n, int32_t k, int32_t dtype);

@@ -70,6 +70,18 @@ def test_absent_parts(lib):
     assert hm.HW_MOE_CORRECTION not in spec.slots[0] and hm.HW_IN_CONV not in spec.slots[0]
 
 
+def test_shared_expert_of_the_experts_size_joins_the_grouped_matrices(lib):
+    from candle_vllm_amd import hybrid_model as hm
+    cfg = _cfg()
+    cfg["layers"][0]["mlp"]["shared"] = {"ff": 12}
+    W = K.random_kerolorn(np.random.default_rng(0), cfg)
+    spec = hm.KerolornSpec(cfg, {k: v.shape for k, v in W.items()})
+    s0 = spec.slots[0]
+    assert s0[hm.HW_MOE_GATE_UP][-2:] == ["l0.mlp.shared.gate", "l0.mlp.shared.up"] and len(s0[hm.HW_MOE_GATE_UP]) == 12
+    assert s0[hm.HW_MOE_DOWN][-1] == "l0.mlp.shared.down" and hm.HW_MLP_GATE_UP not in s0 and hm.HW_MLP_DOWN not in s0
+    assert s0[hm.HW_MOE_ROUTER] == ["l0.mlp.router", "l0.mlp.shared.sg"]
+
+
 def test_registry_knows_the_design_and_its_component(lib):
     from candle_vllm_amd import registry
     assert "Kerolorn" in registry.registered()

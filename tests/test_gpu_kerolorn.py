@@ -239,14 +239,20 @@ def test_router_softmax_correction_choice_and_weights(lib, dtype, T, W, E, top, 
     ids, wts, sg = torch.zeros((T, top), dtype=torch.int32, device="cuda"), torch.zeros((T, top), device="cuda"), torch.zeros(T, device="cuda")
     xn = empty_dt((T, W), dtype)
     ok(lib.mi355_hyb_moe_route(ids.data_ptr(), wts.data_ptr(), sg.data_ptr(), xn.data_ptr(), dtype, P(x), P(nw), P(wr), P(corr),
-                               P(gate) if shared else None, T, W, E, top, 1.7, 1e-5, _st()))
+                               P(gate) if shared else None, T, W, E, top, 1.7, 1e-5, 0, _st()))
     assert np.array_equal(ids.cpu().numpy(), idx)
     assert np.abs(wts.cpu().numpy() - wt).max() < 2e-6 * 1.7
     assert np.abs(host_dt(xn, dtype) - h).max() < (2e-6 if dtype == F32 else 8e-3) * np.abs(h).max()
     if shared:
         assert np.abs(sg.cpu().numpy() - H.sigmoid(h @ gate)).max() < 2e-6
+    if shared:                                                               # the shared expert as one more pair of every token
+        ids2, wts2 = torch.zeros((T, top + 1), dtype=torch.int32, device="cuda"), torch.zeros((T, top + 1), device="cuda")
+        ok(lib.mi355_hyb_moe_route(ids2.data_ptr(), wts2.data_ptr(), None, None, dtype, P(x), P(nw), P(wr), P(corr), P(gate), T, W, E, top, 1.7,
+                                   1e-5, 1, _st()))
+        assert np.array_equal(ids2.cpu().numpy(), np.concatenate([idx, np.full((T, 1), E)], axis=1))
+        assert np.abs(wts2.cpu().numpy() - np.concatenate([wt, H.sigmoid(h @ gate)[:, None]], axis=1)).max() < 4e-6
     # without a norm in front and without a correction
-    ok(lib.mi355_hyb_moe_route(ids.data_ptr(), wts.data_ptr(), None, None, dtype, P(h), None, P(wr), None, None, T, W, E, top, 1.0, 1e-5, _st()))
+    ok(lib.mi355_hyb_moe_route(ids.data_ptr(), wts.data_ptr(), None, None, dtype, P(h), None, P(wr), None, None, T, W, E, top, 1.0, 1e-5, 0, _st()))
     assert np.array_equal(ids.cpu().numpy(), plain)
 
 
@@ -326,7 +332,8 @@ def small_config(variant):
     # sizes that take the matrix-core kernels (attention tiles, 64- and 128-row expert blocks)
     a = {"dim": 64, "heads": 4, "kv_heads": 2, "vdim": 32, "scale": 0.15, "mask": {"keep_first": 5, "size": 70},
          "rot": {"base": 5e5, "dims": 32, "scaling": {"factor": 4.0, "fast": 20.0, "original": 256, "slow": 1.5}}}
-    layers = [{"type": "attention", "mixer": a, "mlp": _moe(8, 2, 64, 32, 2.25)}, {"type": "attention", "mixer": a, "mlp": _moe(2, 1, 32, 96, 1.0)}]
+    # (a shared expert of the experts' size joins the grouped products; one of another size runs as dense products)
+    layers = [{"type": "attention", "mixer": a, "mlp": _moe(8, 2, 64, 64, 2.25)}, {"type": "attention", "mixer": a, "mlp": _moe(2, 1, 32, 96, 1.0)}]
     return {"architecture": "Kerolorn", "canon": {"taps": 4}, "layers": layers, "logit_scale": 0.5, "norm": {"eps": 1e-5}, "vocab": 120, "width": 128}
 
 
@@ -675,3 +682,67 @@ def test_random_configurations_whole_and_mixed_schedules(lib, seed):
         for i in range(3):
             assert row_err(np.concatenate(got[i]), want[i]) < TOL[dtype], (dtype, "schedule", i)
         assert eng.free_pages() == eng.num_blocks and eng.be.state_free_slots() == 4
+
+
+# ------------------------------------------------------------------------------------------------------------ the trace runner
+def _write_model(folder, cfg, W):
+    """config.json + model.safetensors (bf16; 8-byte header length, JSON header, data) of a configuration"""
+    import json
+    import struct
+    head, blobs, at = {}, [], 0
+    for name, a in W.items():
+        raw = bits(a).tobytes()
+        head[name] = {"dtype": "BF16", "shape": list(np.shape(a)), "data_offsets": [at, at + len(raw)]}
+        blobs.append(raw)
+        at += len(raw)
+    hb = json.dumps(head).encode()
+    (folder / "model.safetensors").write_bytes(struct.pack("<Q", len(hb)) + hb + b"".join(blobs))
+    (folder / "config.json").write_text(json.dumps(cfg))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_runner_replays_a_mixed_schedule_from_a_checkpoint_folder(lib, tmp_path, dtype):
+    """bin/trace_run as a user starts it: a folder with config.json and model.safetensors of a configuration of other sizes, steps on
+    standard input -- six requests over time, at most four alive, portions beside single tokens, a pool that only fits because ended
+    requests give their pages and slots back -- and the logits it writes equal the oracle's for every request alone"""
+    _gpu()
+    import json
+    import os
+    import subprocess
+    import sys
+    cfg = small_config(0)
+    rng = np.random.default_rng(17)
+    W = K.random_kerolorn(rng, cfg)
+    if dtype == "bfloat16":
+        settle_router(W, rng)
+    _write_model(tmp_path, cfg, W)
+    lens = {"a": 150, "b": 40, "c": 3, "d": 90, "e": 61, "f": 130}
+    toks = {r: oracle_logits(cfg, W, rng.integers(0, cfg["vocab"], n).tolist(), rng)[2] for r, n in lens.items()}
+    want = {r: K.KerolornOracle(cfg, W).feed(toks[r])[0] for r in toks}
+    sched = [[("a", 70), ("b", 2)], [("a", 1), ("b", 30), ("c", 3)], [("a", 64), ("b", 1), ("d", 65)], [("a", 1), ("b", 7), ("d", 1), ("e", 17)],
+             [("a", 14), ("d", 24), ("e", 1), ("f", 2)], [("e", 43), ("f", 100)], [("f", 1)], [("f", 27)]]
+    at, steps, rows = {r: 0 for r in toks}, [], []
+    for n, step in enumerate(sched):
+        entries, end, got = [], [], []
+        for r, c in step:
+            w = sorted(set([0, c - 1] + rng.integers(0, c, 3).tolist()))
+            entries.append({"id": r, "tokens": toks[r][at[r]:at[r] + c], "want": w})
+            got += [(r, at[r] + k) for k in w]
+            at[r] += c
+            if at[r] == lens[r]:
+                end.append(r)
+        steps.append(json.dumps({"step": n, "entries": entries, "end": end}))
+        rows.append(got)
+    assert at == lens
+    out = tmp_path / "out"
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    # live at any time: a, b, c, d (64-token pages: 192 + 64 + 64 + 128), then e and f in what comes back
+    r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", str(tmp_path), "--dtype", dtype, "--out", str(out),
+                        "--max-tokens", "448"], input="\n".join(steps) + "\n", capture_output=True, text=True, timeout=170)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [l for l in r.stdout.splitlines() if l.startswith("done ")] == ["done %d" % n for n in range(len(sched))]
+    V_ = cfg["vocab"]
+    for n, got in enumerate(rows):
+        a = np.fromfile(out / ("%d.f32" % n), "<f4").reshape(len(got), V_)
+        ref = np.stack([want[r_][p_] for r_, p_ in got])
+        assert row_err(a, ref) < TOL[dtype], (n, dtype)
