@@ -239,7 +239,7 @@ def run_size(name, T=2048, B=8, ctx=2048, dec_steps=16, design="sogodra"):
     def decode_h():
         for _ in range(dec_steps):
             for r in ids:
-                eng.feed(r, [1])
+                eng.feed(r, [int(rng.integers(0, s["vocab"]))])          # (a mixture of experts routes by token: no two sequences the same one)
             eng.step(ids)
     dt = time_calls(decode_h, sync, reps=3)
     out["hybrid_decode_tok_s"] = round(B * dec_steps / dt, 1)

@@ -405,6 +405,7 @@ _sig("mi355_hyb_gather_group_norm", ctypes.c_int, [c_vp, c_i32, c_vp, c_vp, c_vp
 _sig("mi355_hyb_gelu_glu", ctypes.c_int, [c_vp, c_i32, c_vp, c_i32, c_i32, c_i64])
 _sig("mi355_hyb_conv", ctypes.c_int, [c_vp, c_vp, c_i32, c_i32, c_vp, c_vp, c_i64, c_vp, c_vp, c_vp, c_vp] + [c_i32] * 5 + [c_i64])
 _sig("mi355_hyb_pre_norm", ctypes.c_int, [c_vp, c_i32, c_vp, c_vp, c_i32, c_i32, c_f32, c_i64])
+_sig("mi355_hyb_norm_conv", ctypes.c_int, [c_vp, c_i32, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_vp, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_i32, c_f32, c_i64])
 _sig("mi355_hyb_conv_residual", ctypes.c_int, [c_vp, c_i32, c_vp, c_i32, c_i32, c_vp, c_vp, c_i64, c_vp, c_vp, c_vp, c_vp] + [c_i32] * 4 + [c_i64])
 _sig("mi355_hyb_attn_prepare_ex", ctypes.c_int, [c_vp] * 4 + [c_i32] * 4 + [c_vp] * 6 + [c_i32] * 8 + [c_vp, c_f32, c_i32, c_i64])
 _sig("mi355_hyb_masked_attention", ctypes.c_int, [c_vp, c_i32, c_i32, c_i32] + [c_vp] * 8 + [c_i32] * 10 + [c_f32, c_f32, c_i32, c_i32, c_f32,

@@ -1114,6 +1114,60 @@ __global__ void conv_state_update_kernel(ConvArgs p, int n_seqs) {
     for (int j = 0; j < keep; ++j) stt[j] = nv[j];
 }
 
+// The norm in front of a mixer and the convolution added to the mixer's input in one launch: h = x / rms(x) w (nw NULL: h = x),
+// out = h + conv(h).  A workgroup per token recomputes the norms of the TAPS - 1 rows before it that lie in the same portion (the rows
+// before the portion come from the state slot, zeros before position 0).  hn != NULL receives h (what conv_state_update_kernel then
+// reads); update: every sequence of the step brings ONE token, and the token's workgroup moves the slot's rows itself (a thread reads
+// and writes its own channels only).
+struct NormConvArgs {
+    float* out; uint16_t* out_bf16; float* hn; const float* x; const float* nw; const float* cw; float* state; int64_t state_stride;
+    const uint32_t* ctx; const uint32_t* cu_q; const int32_t* slots; const int32_t* tok_seq; int W, update; float eps;
+};
+template <int TAPS, int NW> __global__ __launch_bounds__(64 * NW) void norm_conv_kernel(NormConvArgs p) {
+    __shared__ float red[TAPS][NW];
+    __shared__ float inv_s[TAPS];
+    const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int s = p.tok_seq[t], cs = (int)p.cu_q[s];
+    const int start_pos = (int)p.ctx[s] - (int)(p.cu_q[s + 1] - p.cu_q[s]);
+    if (p.nw) {
+        float ss[TAPS];
+#pragma unroll
+        for (int j = 0; j < TAPS; ++j) {
+            ss[j] = 0.f;
+            const int o = t - (TAPS - 1 - j);
+            if (o >= cs)
+                for (int i = threadIdx.x; i < p.W; i += 64 * NW) { const float v = p.x[(size_t)o * p.W + i]; ss[j] = fmaf(v, v, ss[j]); }
+        }
+#pragma unroll
+        for (int j = 0; j < TAPS; ++j) { ss[j] = wave_sum(ss[j]); if (lane == 0) red[j][wave] = ss[j]; }
+        __syncthreads();
+        if (threadIdx.x < TAPS) {
+            float sum = 0.f;
+#pragma unroll
+            for (int w = 0; w < NW; ++w) sum += red[threadIdx.x][w];
+            inv_s[threadIdx.x] = 1.f / sqrtf(sum / (float)p.W + p.eps);
+        }
+        __syncthreads();
+    }
+    float* stt = p.state + (size_t)p.slots[s] * p.state_stride;
+    for (int i = threadIdx.x; i < p.W; i += 64 * NW) {
+        float h[TAPS], acc = 0.f;
+#pragma unroll
+        for (int j = 0; j < TAPS; ++j) {
+            const int o = t - (TAPS - 1 - j);
+            if (o >= cs) h[j] = p.nw ? p.x[(size_t)o * p.W + i] * inv_s[j] * p.nw[i] : p.x[(size_t)o * p.W + i];
+            else { const int back = cs - o; h[j] = (start_pos > 0 && start_pos - back >= 0) ? stt[(size_t)i * (TAPS - 1) + (TAPS - 1 - back)] : 0.f; }
+            acc = fmaf(p.cw[(size_t)i * TAPS + j], h[j], acc);
+        }
+        acc += h[TAPS - 1];
+        if (p.out_bf16) p.out_bf16[(size_t)t * p.W + i] = f32_to_bf16(acc); else p.out[(size_t)t * p.W + i] = acc;
+        if (p.hn) p.hn[(size_t)t * p.W + i] = h[TAPS - 1];
+        if (p.update)
+#pragma unroll
+            for (int j = 0; j + 1 < TAPS; ++j) stt[(size_t)i * (TAPS - 1) + j] = h[j + 1];
+    }
+}
+
 // ------------------------------------------------------------------------------------------------------------ gated delta rule
 struct DeltaArgs {
     float* o; float* state; int64_t state_stride;
@@ -2210,6 +2264,28 @@ int mi355_hyb_moe_combine_norm_add(float* x, void* xcopy, const float* y_rows, c
         moe_combine_norm_add_kernel<true><<<T, 256, lds, to_stream(stream)>>>(x, (uint16_t*)xcopy, y_rows, pos, weights, y_shared, shared_gate, w, width, top, eps);
     else
         moe_combine_norm_add_kernel<false><<<T, 256, lds, to_stream(stream)>>>(x, (uint16_t*)xcopy, y_rows, pos, weights, y_shared, shared_gate, w, width, top, eps);
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_norm_conv(void* out, int32_t out_dtype, float* hn, const float* x, const float* norm_w, const float* conv_w, float* conv_state,
+                        int64_t state_stride, const uint32_t* context_lens, const uint32_t* cu_seqlens_q, const int32_t* state_slots,
+                        const int32_t* tok_seq, int32_t num_seqs, int32_t T, int32_t width, int32_t taps, int32_t update_state, float eps,
+                        int64_t stream) {
+    if (!out || !x || !conv_w || !conv_state || !context_lens || !cu_seqlens_q || !state_slots || !tok_seq || !is_dt(out_dtype)) return -1;
+    if (width <= 0 || taps < 1 || taps > 8) return -1;
+    if (update_state && T != num_seqs) return -1;                       // a workgroup moves its slot's rows only when it is the portion
+    if (T <= 0) return 0;
+    const bool f = out_dtype == MI355_DTYPE_F32;
+    NormConvArgs p{f ? (float*)out : nullptr, f ? nullptr : (uint16_t*)out, hn, x, norm_w, conv_w, conv_state, state_stride, context_lens,
+                   cu_seqlens_q, state_slots, tok_seq, width, update_state ? 1 : 0, eps};
+    hipStream_t s_ = to_stream(stream);
+    // few tokens (decoding batches): sixteen waves per token, so that a thread walks one or two channels instead of eight
+#define NC(TAPS) do { if (T <= 64) norm_conv_kernel<TAPS, 16><<<T, 1024, 0, s_>>>(p); else norm_conv_kernel<TAPS, 4><<<T, 256, 0, s_>>>(p); } while (0)
+    switch (taps) {
+        case 1: NC(1); break; case 2: NC(2); break; case 3: NC(3); break; case 4: NC(4); break;
+        case 5: NC(5); break; case 6: NC(6); break; case 7: NC(7); break; default: NC(8); break;
+    }
+#undef NC
     LAUNCH_OK(); return 0;
 }
 

@@ -501,13 +501,25 @@ static int forward_enqueue(HModel* m, const uint32_t* tokens, const int64_t* pos
         const int ldp = L.in_rows;
         const void* min_ = xin;                                         // the mixer's input
         if (c.in_conv) {
-            // h + conv(h): h = the normed x (form 2; f32 in m->y, free until the output projection) or x itself
-            const float* h = m->x;
-            if (sandwich) { HCHECK(mi355_hyb_pre_norm(m->y, MI355_DTYPE_F32, m->x, f(MI355_HW_PRE_NORM1), T, W, eps, stream)); h = m->y; }
+            // h + conv(h): h = the normed x (form 2) or x itself.  Up to 8 taps: norm, convolution (and, when every sequence brings one
+            // token, the move of the slot's rows) are one launch; else the normed rows go through m->y (free until the output projection)
             float* cst = m->state + L.in_conv_off;
-            HCHECK(mi355_hyb_conv_residual(m->pre, dt, h, W, 0, f(MI355_HW_IN_CONV), cst, m->slot_floats, context_lens, cu_seqlens_q, state_slots,
-                                           m->tok_seq, num_seqs, T, W, c.in_conv, stream));
-            HCHECK(mi355_hyb_conv_state_update(cst, m->slot_floats, h, W, 0, context_lens, cu_seqlens_q, state_slots, num_seqs, W, c.in_conv, stream));
+            const float* nw = sandwich ? f(MI355_HW_PRE_NORM1) : nullptr;
+            if (c.in_conv <= 8) {
+                const int self_update = T == num_seqs;
+                HCHECK(mi355_hyb_norm_conv(m->pre, dt, (sandwich && !self_update) ? m->y : nullptr, m->x, nw, f(MI355_HW_IN_CONV), cst, m->slot_floats,
+                                           context_lens, cu_seqlens_q, state_slots, m->tok_seq, num_seqs, T, W, c.in_conv, self_update, eps, stream));
+                if (!self_update)
+                    HCHECK(mi355_hyb_conv_state_update(cst, m->slot_floats, sandwich ? m->y : m->x, W, 0, context_lens, cu_seqlens_q, state_slots,
+                                                       num_seqs, W, c.in_conv, stream));
+            } else {
+                const float* h = m->x;
+                if (sandwich) { HCHECK(mi355_hyb_pre_norm(m->y, MI355_DTYPE_F32, m->x, nw, T, W, eps, stream)); h = m->y; }
+                HCHECK(mi355_hyb_conv_residual(m->pre, dt, h, W, 0, f(MI355_HW_IN_CONV), cst, m->slot_floats, context_lens, cu_seqlens_q,
+                                               state_slots, m->tok_seq, num_seqs, T, W, c.in_conv, stream));
+                HCHECK(mi355_hyb_conv_state_update(cst, m->slot_floats, h, W, 0, context_lens, cu_seqlens_q, state_slots, num_seqs, W, c.in_conv,
+                                                   stream));
+            }
             min_ = m->pre;
         } else if (sandwich) {
             HCHECK(mi355_hyb_pre_norm(m->pre, dt, m->x, f(MI355_HW_PRE_NORM1), T, W, eps, stream));

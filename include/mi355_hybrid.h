@@ -269,6 +269,13 @@ int mi355_hyb_conv_residual(void* out, int32_t out_dtype, const float* in, int32
                             const float* conv_state, int64_t state_stride, const uint32_t* context_lens, const uint32_t* cu_seqlens_q,
                             const int32_t* state_slots, const int32_t* token_seq, int32_t num_seqs, int32_t num_tokens, int32_t channels,
                             int32_t taps, int64_t stream);
+/* the two above in ONE launch for taps <= 8: h = RMS norm of x times norm_w (norm_w NULL: h = x), out (dt_out) [T, width] = h + conv(h).
+ * hn: NULL, or f32 [T, width] that receives h (what mi355_hyb_conv_state_update then reads).  update_state != 0 (only when every
+ * sequence brings one token, T == num_seqs): the kernel moves the state behind the token itself and no update launch is needed */
+int mi355_hyb_norm_conv(void* out, int32_t out_dtype, float* hn, const float* x, const float* norm_w, const float* conv_w, float* conv_state,
+                        int64_t state_stride, const uint32_t* context_lens, const uint32_t* cu_seqlens_q, const int32_t* state_slots,
+                        const int32_t* token_seq, int32_t num_seqs, int32_t num_tokens, int32_t width, int32_t taps, int32_t update_state,
+                        float eps, int64_t stream);
 /* mi355_hyb_attn_prepare with the remaining switches: interleaved = rotated pairs are (2i, 2i + 1); norm_mode 0 = none, 1 = RMS norm
  * with weights before the rotation (q_norm_w / k_norm_w, NULL = no weight), 2 = RMS norm without a weight AFTER the rotation;
  * q_head_scale f32 [heads] or NULL: head h's query is multiplied by it (a temperature per head folded into the query) */

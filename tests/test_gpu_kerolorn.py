@@ -104,6 +104,26 @@ def test_pre_norm_and_input_convolution_over_portions(lib, dtype, taps, C):
         got.append(host_dt(out, dtype))
         lo += n
     assert np.abs(np.concatenate(got) - want).max() < (2e-5 if dtype == F32 else 2e-2) * max(1.0, np.abs(want).max())
+    # norm, convolution and (for single tokens) the move of the state in ONE launch: the same result, the same state
+    state2 = dev(rng.standard_normal((n_slots, stride)))
+    lo, got2 = 0, []
+    for n in (1, 2, 1, 7, 1, 11):
+        seq = torch.zeros(n, dtype=torch.int32, device="cuda")
+        hn = torch.zeros((n, C), device="cuda")
+        out = empty_dt((n, C), dtype)
+
+        def args():
+            return P([lo + n], np.int32), P([0, n], np.int32), P([2], np.int32)
+        own = int(n == 1)
+        ok(lib.mi355_hyb_norm_conv(out.data_ptr(), dtype, None if own else hn.data_ptr(), P(x[lo:lo + n]), P(nw), P(w), state2.data_ptr(), stride,
+                                   *args(), seq.data_ptr(), 1, n, C, taps, own, 1e-5, _st()))
+        if not own:
+            ok(lib.mi355_hyb_conv_state_update(state2.data_ptr(), stride, hn.data_ptr(), C, 0, *args(), 1, C, taps, _st()))
+        got2.append(host_dt(out, dtype))
+        lo += n
+    assert np.abs(np.concatenate(got2) - want).max() < (2e-5 if dtype == F32 else 2e-2) * max(1.0, np.abs(want).max())
+    if taps > 1:
+        assert np.abs(state2.cpu().numpy()[2, :C * (taps - 1)] - state.cpu().numpy()[2, :C * (taps - 1)]).max() < 1e-5
     # the rounded norm as the product's operand
     out = empty_dt((T, C), BF16)
     ok(lib.mi355_hyb_pre_norm(out.data_ptr(), BF16, P(x), P(nw), T, C, 1e-5, _st()))
