@@ -284,8 +284,8 @@ int mi355_hyb_attn_prepare_ex(void* q_out, void* k_pages, void* v_pages, const f
                               const int64_t* positions, const int64_t* slot_mapping, int32_t num_tokens, int32_t heads,
                               int32_t kv_heads, int32_t dim, int32_t vdim, int32_t rot_dims, int32_t interleaved, int32_t norm_mode,
                               const float* q_head_scale, float eps, int32_t dtype, int64_t stream);
-/* mi355_hyb_window_attention_ex with kept first tokens: a query at position i sees key j when j <= i and (window == 0 or
- * i - j < window or j < keep_first); kept keys keep their own positions */
+/* mi355_hyb_window_attention_ex with kept first tokens: beside the keys inside its window (all earlier keys when window == 0) a query
+ * sees the keys at positions below keep_first; those keep their own positions and rotations */
 int mi355_hyb_masked_attention(void* out, int32_t out_dtype, int32_t ldo, int32_t out_off, const void* q, const void* k_pages,
                                const void* v_pages, const uint32_t* block_tables, const uint32_t* context_lens,
                                const uint32_t* cu_seqlens_q, const int32_t* token_seq, const float* sink, int32_t num_seqs,

@@ -39,7 +39,8 @@ def unit_rms(x, eps):
 
 
 def window_keep_mask(q_pos, k_pos, window, keep_first):
-    """query at i sees key at j when j <= i and (i - j < window or j < keep_first); window 0 = no window"""
+    """bool [queries, keys]: causal; with a window (0 = none) only the last `window` positions stay visible -- and the keys at
+    positions below keep_first, whatever their distance"""
     i, j = np.asarray(q_pos)[:, None], np.asarray(k_pos)[None, :]
     vis = j <= i
     if window:
