@@ -563,6 +563,25 @@ def test_long_decoding_and_first_tokens(lib):
     assert row_err(np.concatenate(rows), want) < TOL["float32"]
 
 
+def test_more_taps_than_the_single_launch_takes(lib):
+    """ten taps: the norm, the convolution and the move of its state run as three launches; portions shorter than the taps and single
+    tokens continue from the slot"""
+    _gpu()
+    from candle_vllm_amd.step_engine import StepEngine
+    cfg = dict(small_config(0), canon={"taps": 10})
+    m, W = build(cfg, "float32", seed=14)
+    rng = np.random.default_rng(15)
+    toks = rng.integers(0, cfg["vocab"], 60).tolist()
+    want, _, toks = oracle_logits(cfg, W, toks, rng)
+    eng = StepEngine(m, 64)
+    lo, rows = 0, []
+    for c in [3, 1, 1, 12, 2, 9, 1, 1, 1, 29]:
+        eng.feed("a", toks[lo:lo + c])
+        rows.append(eng.step(["a"], [list(range(c))]).cpu().numpy())
+        lo += c
+    assert lo == 60 and row_err(np.concatenate(rows), want) < TOL["float32"]
+
+
 def test_graph_replays_equal_eager_steps(lib):
     """decoding batches replay a captured hipGraph: every replay, with eager prompt portions of other requests between them, gives the
     eager step's logits bit for bit"""
