@@ -1723,6 +1723,7 @@ __global__ void scale_f32_kernel(float* x, float s, int64_t n) {
     if (i < n) x[i] *= s;
 }
 
+int g_attn_wider = 1;           // A/B: twelve waves per (token, head) for the smallest decoding batches
 int g_attn_group = 1;           // 0: grouped-query prompt steps take the kernel with one wave per head (A/B, tests of both paths)
 int g_attn_mfma = 1;            // mi355_hyb_set_attention_mfma(0): prompt steps take the generic kernel too (A/B, tests of both paths)
 
@@ -1739,7 +1740,7 @@ int mi355_hyb_token_seq(int32_t* tok_seq, const uint32_t* cu_seqlens_q, int32_t 
     token_seq_kernel<<<num_seqs, 64, 0, to_stream(stream)>>>(tok_seq, cu_seqlens_q, num_seqs);
     LAUNCH_OK(); return 0;
 }
-void mi355_hyb_set_attention_mfma(int32_t on) { g_attn_mfma = on ? 1 : 0; g_attn_group = on == 2 ? 0 : 1; }
+void mi355_hyb_set_attention_mfma(int32_t on) { g_attn_mfma = on ? 1 : 0; g_attn_group = on == 2 ? 0 : 1; g_attn_wider = on == 3 ? 0 : 1; }
 int mi355_hyb_bf16_to_f32(float* out, const uint16_t* in, int64_t n, int64_t stream) {
     if (n <= 0) return 0;
     bf16_to_f32_kernel<<<(unsigned)((n + 255) / 256), 256, 0, to_stream(stream)>>>(out, in, n);
@@ -1955,15 +1956,17 @@ int mi355_hyb_masked_attention(void* out, int32_t out_dtype, int32_t ldo, int32_
     }
     // few (token, head) pairs (decoding batches): eight waves share a window instead of four
     const bool wide = (int64_t)T * heads < 2048;
+    // a handful of sequences: twelve waves (a window of a thousand keys plus kept tokens is two rounds of 64-key chunks instead of three)
+    const bool wider = (int64_t)T * heads <= 256 && g_attn_wider;
     // cross mode with 16-byte rows: 4 or 2 value heads per workgroup, the rest of the key/value heads along z
     int nv = (cross && vec) ? (kv_heads % 4 == 0 ? 4 : kv_heads % 2 == 0 ? 2 : 1) : 1;
-    if ((size_t)8 * nv * vdim * sizeof(float) > 32768) nv = 1;          // the waves' partial sums must fit the workgroup's LDS
+    if ((size_t)(wider ? 12 : 8) * nv * vdim * sizeof(float) > 32768) nv = 1;          // the waves' partial sums must fit the workgroup's LDS
     while (nv > 1 && (int64_t)T * heads * (nz / nv) < 512) nv >>= 1;    // decoding batches: rather more workgroups than shared scores
     const dim3 ggrid(T, heads, nz / nv);
 #define WA4(TC, NW, VEC, DQ, NV) window_attention_kernel<TC, NW, VEC, DQ, NV><<<ggrid, 64 * NW, (size_t)(((dim + 3) & ~3) + 2 * NW + NW * NV * vdim) * sizeof(float), s_>>>(p)
 #define WA3(TC, NW, VEC, DQ) do { if (nv == 4) WA4(TC, NW, VEC, DQ, 4); else if (nv == 2) WA4(TC, NW, VEC, DQ, 2); else WA4(TC, NW, VEC, DQ, 1); } while (0)
 #define WA2(TC, NW) do { if (!vec) WA4(TC, NW, false, 0, 1); else WA3(TC, NW, true, 0); } while (0)
-#define WA(TC) do { if (wide) WA2(TC, 8); else WA2(TC, 4); } while (0)
+#define WA(TC) do { if (wider) WA2(TC, 12); else if (wide) WA2(TC, 8); else WA2(TC, 4); } while (0)
     if (f) WA(float); else WA(uint16_t);
 #undef WA
 #undef WA2
