@@ -345,14 +345,18 @@ class HybridLayer(ctypes.Structure):
                 ("a_rot_interleaved", c_i32), ("a_kv_rank", c_i32), ("a_rot_dim", c_i32), ("a_head_gate", c_i32), ("a_conv", c_i32),
                 ("a_norm_whole", c_i32), ("a_v_unit", c_i32), ("a_softcap", c_f32), ("a_talk", c_i32), ("share_with", c_i32),
                 ("a_keep_first", c_i32), ("a_norm_after_rot", c_i32), ("a_head_temp", c_i32), ("in_conv", c_i32),
-                ("moe_experts", c_i32), ("moe_top", c_i32), ("moe_shared_ff", c_i32), ("moe_scale", c_f32)]
+                ("moe_experts", c_i32), ("moe_top", c_i32), ("moe_shared_ff", c_i32), ("moe_scale", c_f32),
+                ("moe_sigmoid", c_i32), ("moe_groups", c_i32), ("moe_keep_groups", c_i32), ("moe_normalise", c_i32),
+                ("d_norm_groups", c_i32), ("a_dist_bias", c_i32), ("a_q_rank", c_i32), ("a_out_gate", c_i32), ("kv_from", c_i32),
+                ("side_dim", c_i32), ("side_col", c_i32), ("depth_terms", c_i32)]
 
 
 class HybridConfig(ctypes.Structure):
     """mirror of `mi355_hybrid_config`"""
     _fields_ = [("width", c_i32), ("vocab", c_i32), ("n_layers", c_i32), ("dtype", c_i32), ("block_size", c_i32),
                 ("state_slots", c_i32), ("norm_eps", c_f32), ("unit_eps", c_f32),
-                ("residual_form", c_i32), ("resid_alpha", c_f32), ("norm_groups", c_i32), ("logit_scale", c_f32)]
+                ("residual_form", c_i32), ("resid_alpha", c_f32), ("norm_groups", c_i32), ("logit_scale", c_f32),
+                ("norm_kind", c_i32), ("embed_scale", c_f32), ("logit_softcap", c_f32), ("tie_head", c_i32), ("side_cols", c_i32)]
 
 
 _sig("mi355_be_state_init", c_i32, [c_vp, c_i32])
@@ -417,6 +421,24 @@ _sig("mi355_hyb_linear_grouped", ctypes.c_int, [c_vp, c_i32, c_vp, c_i32, c_i32,
 _sig("mi355_hyb_silu_glu", ctypes.c_int, [c_vp, c_i32, c_vp, c_i32, c_i32, c_vp, c_i32, c_i64])
 _sig("mi355_hyb_moe_combine_norm_add", ctypes.c_int, [c_vp] * 8 + [c_i32, c_i32, c_i32, c_f32, c_i64])
 _sig("mi355_hyb_scale_f32", ctypes.c_int, [c_vp, c_f32, c_i64, c_i64])
+_sig("mi355_hyb_embed_scaled", ctypes.c_int, [c_vp, c_vp, c_vp, c_i32, c_i32, c_i32, c_f32, c_i32, c_i64])
+_sig("mi355_hyb_pre_norm_ex", ctypes.c_int, [c_vp, c_i32, c_vp, c_vp, c_i32, c_vp, c_i32, c_i32, c_i32, c_f32, c_i64])
+_sig("mi355_hyb_gather_norm_ex", ctypes.c_int, [c_vp, c_i32, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32, c_f32, c_i64])
+_sig("mi355_hyb_add2", ctypes.c_int, [c_vp, c_vp, c_vp, c_i64, c_i64])
+_sig("mi355_hyb_moe_combine_add", ctypes.c_int, [c_vp] * 5 + [c_i32, c_i32, c_i32, c_i64])
+_sig("mi355_hyb_relu2", ctypes.c_int, [c_vp, c_i32, c_vp, c_i64, c_i64])
+_sig("mi355_hyb_tanh_cap", ctypes.c_int, [c_vp, c_f32, c_i64, c_i64])
+_sig("mi355_hyb_elem_gate", ctypes.c_int, [c_vp, c_i32, c_vp, c_vp, c_i32, c_i32, c_i32, c_i64])
+_sig("mi355_hyb_side_act", ctypes.c_int, [c_vp, c_i32, c_vp, c_vp, c_i32, c_i32, c_vp, c_i32, c_i32, c_i32, c_i32, c_i64])
+_sig("mi355_hyb_depth_average", ctypes.c_int, [c_vp, c_vp, c_vp, c_i32, c_i64, c_i64])
+_sig("mi355_hyb_gate_group_norm", ctypes.c_int, [c_vp, c_i32, c_vp, c_vp, c_i32, c_vp, c_i32, c_i32, c_i32, c_f32, c_i64])
+_sig("mi355_hyb_ssd_scan", ctypes.c_int, [c_vp, c_vp, c_i64, c_vp, c_i32, c_vp, c_i32] + [c_vp] * 6 + [c_i32] * 6 + [c_i64])
+_sig("mi355_hyb_conv_bias", ctypes.c_int, [c_vp, c_vp, c_i32, c_i32, c_vp, c_vp, c_vp, c_i64, c_vp, c_vp, c_vp, c_vp] + [c_i32] * 5 + [c_i64])
+_sig("mi355_hyb_biased_attention", ctypes.c_int, [c_vp, c_i32, c_i32, c_i32] + [c_vp] * 9 + [c_i32] * 10 + [c_f32, c_f32, c_i32, c_i32, c_f32,
+                                                                                                     c_i32, c_i32, c_i64])
+_sig("mi355_hyb_latent_prepare_ex", ctypes.c_int, [c_vp, c_vp, c_vp, c_i32, c_i32, c_vp, c_i32, c_i32] + [c_vp] * 6 + [c_i32] * 7 + [c_f32, c_i32, c_i64])
+_sig("mi355_hyb_moe_route_ex", ctypes.c_int, [c_vp, c_vp, c_vp, c_vp, c_i32, c_vp, c_vp, c_vp, c_vp, c_vp, c_i32, c_i32, c_i32, c_i32, c_f32, c_f32,
+                                                c_i32, c_i32, c_i32, c_i32, c_i32, c_i64])
 
 # the hand-written ctypes mirrors must have the layout the library was built with
 for _id, _cls in ((0, QmmDesc), (1, LlamaConfig), (2, DenseConfig), (3, RopeScaling), (4, HybridConfig), (5, HybridLayer)):

@@ -10,30 +10,10 @@
 #include <math.h>
 
 #include "common.h"
+#include "hybrid_device.h"
 #include "../../include/mi355_hybrid.h"
 
 namespace {
-
-template <typename T> __device__ __forceinline__ float ld(const T* p, size_t i);
-template <> __device__ __forceinline__ float ld<float>(const float* p, size_t i) { return p[i]; }
-template <> __device__ __forceinline__ float ld<uint16_t>(const uint16_t* p, size_t i) { return bf16_to_f32(p[i]); }
-template <typename T> __device__ __forceinline__ void st(T* p, size_t i, float v);
-template <> __device__ __forceinline__ void st<float>(float* p, size_t i, float v) { p[i] = v; }
-template <> __device__ __forceinline__ void st<uint16_t>(uint16_t* p, size_t i, float v) { p[i] = f32_to_bf16(v); }
-
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
-    return v;
-}
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o));
-    return v;
-}
-__device__ __forceinline__ float sigmoidf_(float x) { return 1.f / (1.f + expf(-x)); }
-__device__ __forceinline__ float siluf_(float x) { return x / (1.f + expf(-x)); }
-__device__ __forceinline__ float softplusf_(float x) { return x > 20.f ? x : log1pf(expf(x)); }
 
 // ------------------------------------------------------------------------------------------------------------ matrix products
 // 8 consecutive operands of a row as one MFMA fragment (bf16), zero beyond `kend`
@@ -509,7 +489,9 @@ struct AttnArgs {
     int cross;              // blockIdx.z = the key/value head whose VALUES this block sums (scores still against the head's own keys)
     int cpk;                // lanes that share a key row when it is read 16 bytes a lane (power of two >= d / elements per 16 bytes)
     int keep;               // with a window: keys at positions < keep stay visible (the first tokens of the sequence)
+    const float* dist;      // != NULL: [2, H] = r1, r2; score <- score - r1[h] ln(1 + r2[h] (query position - key position))
 };
+__device__ __forceinline__ float dist_bias(float r1, float r2, int d) { return r1 * log1pf(r2 * (float)d); }
 __device__ __forceinline__ float cap_score(float s, float cap) { return cap > 0.f ? cap * tanhf(s / cap) : s; }
 // 16 bytes of a page row as floats (EPV = 8 bf16 or 4 f32)
 template <typename TC> struct Vec16;
@@ -567,6 +549,7 @@ template <typename TC, int NW, bool VEC, int DQ, int NV> __global__ __launch_bou
     float qv[EPV];
 #pragma unroll
     for (int e = 0; e < EPV; ++e) qv[e] = (VEC && qok) ? qs[qchunk * EPV + e] : 0.f;
+    const float r1 = p.dist ? p.dist[h] : 0.f, r2 = p.dist ? p.dist[p.H + h] : 0.f;
     float m = -INFINITY, l = 0.f, acc[NV][NACC];
 #pragma unroll
     for (int n = 0; n < NV; ++n)
@@ -605,12 +588,12 @@ template <typename TC, int NW, bool VEC, int DQ, int NV> __global__ __launch_bou
                     if (lane / kq == u0 + u) dot = v;
                 }
             }
-            if (j <= pos) sc = cap_score(dot * p.scale, p.softcap);
+            if (j <= pos) sc = cap_score(dot * p.scale, p.softcap) - (p.dist ? dist_bias(r1, r2, pos - j) : 0.f);
         } else if (j <= pos) {
             const TC* kr = static_cast<const TC*>(p.k_pages) + (size_t)page_row * p.k_ld + g * p.d;
             float dot = 0.f;
             for (int i = 0; i < p.d; ++i) dot = fmaf(qs[i], ld<TC>(kr, i), dot);
-            sc = cap_score(dot * p.scale, p.softcap);
+            sc = cap_score(dot * p.scale, p.softcap) - (p.dist ? dist_bias(r1, r2, pos - j) : 0.f);
         }
         const float mn = fmaxf(m, wave_max(sc));
         const float pj = (j <= pos) ? expf(sc - mn) : 0.f;
@@ -744,6 +727,7 @@ void window_attention_mfma_kernel(AttnArgs p) {
 #pragma unroll
         for (int c = 0; c < VT; ++c) acc[n][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     const int hi = pos0 + nq - 1;
+    const float r1 = p.dist ? p.dist[h] : 0.f, r2 = p.dist ? p.dist[p.H + h] : 0.f;
     const int lo = p.window > 0 ? max(0, pos0 - p.window + 1) : 0;
     // the keys any query of the tile may see, in one run of indices: the kept first tokens below the lowest window, then [lo, hi]
     const int nkeep = min(p.keep, lo), n_vis = nkeep + hi - lo + 1;
@@ -821,7 +805,7 @@ void window_attention_mfma_kernel(AttnArgs p) {
             for (int kt = 0; kt < 4; ++kt) {
                 const int key = key_at(j0 + kt * 16 + m16);
                 const bool ok_ = r < nq && key <= qpos && (p.window == 0 || qpos - key < p.window || key < p.keep);
-                sc[v][kt] = ok_ ? cap_score(sacc[kt][v] * p.scale, p.softcap) : -INFINITY;
+                sc[v][kt] = ok_ ? cap_score(sacc[kt][v] * p.scale, p.softcap) - (p.dist ? dist_bias(r1, r2, qpos - key) : 0.f) : -INFINITY;
                 mx[v] = fmaxf(mx[v], sc[v][kt]);
             }
 #pragma unroll
@@ -935,6 +919,7 @@ template <int DK, int VT, int HPG> __global__ __launch_bounds__(64 * HPG) void w
 #pragma unroll
     for (int c = 0; c < VT; ++c) acc[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     const int hi = pos0 + nq - 1;
+    const float r1 = p.dist ? p.dist[h] : 0.f, r2 = p.dist ? p.dist[p.H + h] : 0.f;
     const int lo = p.window > 0 ? max(0, pos0 - p.window + 1) : 0;
     const int nkeep = min(p.keep, lo), n_vis = nkeep + hi - lo + 1;
     auto key_at = [&](int i) { return i < nkeep ? i : (i < n_vis ? lo + (i - nkeep) : hi + 1); };
@@ -1004,7 +989,7 @@ template <int DK, int VT, int HPG> __global__ __launch_bounds__(64 * HPG) void w
             for (int kt = 0; kt < 4; ++kt) {
                 const int key = key_at(j0 + kt * 16 + m16);
                 const bool ok_ = r < nq && key <= qpos && (p.window == 0 || qpos - key < p.window || key < p.keep);
-                sc[v][kt] = ok_ ? cap_score(sacc[kt][v] * p.scale, p.softcap) : -INFINITY;
+                sc[v][kt] = ok_ ? cap_score(sacc[kt][v] * p.scale, p.softcap) - (p.dist ? dist_bias(r1, r2, qpos - key) : 0.f) : -INFINITY;
                 mx[v] = fmaxf(mx[v], sc[v][kt]);
             }
 #pragma unroll
@@ -1069,6 +1054,7 @@ struct ConvArgs {
     int act;                // 0 = none, 1 = silu
     int add_input;          // the convolution is added to its own input (h + conv(h))
     uint16_t* out_bf16;     // != NULL: the result goes here as bf16 instead of `out`
+    const float* bias;      // != NULL: added per channel in front of the activation
 };
 __global__ void conv_silu_kernel(ConvArgs p) {
     const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -1090,6 +1076,7 @@ __global__ void conv_silu_kernel(ConvArgs p) {
         acc = fmaf(p.w[(size_t)c * p.taps + i], v, acc);
     }
     if (p.add_input) acc += p.proj[(size_t)t * p.ldp + p.off + c];
+    if (p.bias) acc += p.bias[c];
     acc = p.act ? siluf_(acc) : acc;
     if (p.out_bf16) p.out_bf16[idx] = f32_to_bf16(acc); else p.out[idx] = acc;
 }
@@ -1206,23 +1193,6 @@ __global__ __launch_bounds__(64) void delta_prep_kernel(DeltaArgs p, float* prep
         out[g_off + h] = expf(-a_rate * softplusf_(p.decay_in[(size_t)t * p.ldd + h] + p.dt_bias[h]));
     }
     if (lane == 0) out[b_off + h] = sigmoidf_(p.proj[(size_t)t * p.ldp + p.b_off + h]);
-}
-
-// sum over the LPC neighbouring lanes that share a state column
-// (data-parallel-primitive moves inside a row of 16 lanes: swap inside pairs, swap pairs inside quads, mirror inside half rows,
-// mirror inside the row -- after each add every lane holds the sum of twice as many lanes; no LDS traffic, a few cycles each)
-template <int CTRL> __device__ __forceinline__ float dpp_move(float x) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), CTRL, 0xF, 0xF, true));
-}
-template <int LPC> __device__ __forceinline__ float column_sum(float x) {
-    static_assert(LPC == 4 || LPC == 16, "a column is shared by a quad or by a row of 16 lanes");
-    x += dpp_move<0xB1>(x);                      // quad_perm [1, 0, 3, 2]
-    x += dpp_move<0x4E>(x);                      // quad_perm [2, 3, 0, 1]
-    if (LPC == 16) {
-        x += dpp_move<0x141>(x);                 // row_half_mirror
-        x += dpp_move<0x140>(x);                 // row_mirror
-    }
-    return x;
 }
 
 // The scan.  A workgroup of 256 threads owns 256 / LPC columns of one (sequence, head)'s state S [d, vd]; LPC neighbouring lanes share
@@ -1473,7 +1443,7 @@ template <typename TC> __global__ __launch_bounds__(256) void attn_prepare_whole
 
 struct LatentPrepArgs {
     void* q_out; void* pages;
-    const float* proj; int ldp, q_off, c_off;
+    const float* qsrc; int ldq, q_off; const float* csrc; int ldc, c_off;   // pages NULL: nothing is cached and csrc is not read
     const float* q_abs; const float* cw; const float* cos_t; const float* sin_t;
     const int64_t* positions; const int64_t* slots;
     int H, d, r, rank, rot, interleaved; float eps;
@@ -1493,19 +1463,22 @@ __device__ __forceinline__ float rotated_elem(const float* v, int i, int rot, in
 template <typename TC> __global__ __launch_bounds__(256) void latent_prepare_kernel(LatentPrepArgs p) {
     __shared__ float red[4];
     const int t = blockIdx.x, dq = p.rank + p.r;
-    const float* row = p.proj + (size_t)t * p.ldp;
+    const float* row = p.qsrc + (size_t)t * p.ldq;
     const int64_t pos = p.positions[t], slot = p.slots[t];
     const float* cs = p.cos_t + pos * (p.rot / 2);
     const float* sn = p.sin_t + pos * (p.rot / 2);
-    float ss = 0.f;
-    for (int i = threadIdx.x; i < p.rank; i += blockDim.x) { const float v = row[p.c_off + i]; ss = fmaf(v, v, ss); }
-    ss = block_sum(ss, red);
-    const float inv = 1.f / sqrtf(ss / (float)p.rank + p.eps);
-    if (slot >= 0) {
-        TC* dst = static_cast<TC*>(p.pages) + (size_t)slot * dq;
-        for (int i = threadIdx.x; i < p.rank; i += blockDim.x) st<TC>(dst, i, row[p.c_off + i] * inv * p.cw[i]);
-        const float* kr = row + p.c_off + p.rank;
-        for (int i = threadIdx.x; i < p.r; i += blockDim.x) st<TC>(dst, p.rank + i, rotated_elem(kr, i, p.rot, p.interleaved, cs, sn));
+    if (p.pages) {
+        const float* crow = p.csrc + (size_t)t * p.ldc + p.c_off;
+        float ss = 0.f;
+        for (int i = threadIdx.x; i < p.rank; i += blockDim.x) { const float v = crow[i]; ss = fmaf(v, v, ss); }
+        ss = block_sum(ss, red);
+        const float inv = 1.f / sqrtf(ss / (float)p.rank + p.eps);
+        if (slot >= 0) {
+            TC* dst = static_cast<TC*>(p.pages) + (size_t)slot * dq;
+            for (int i = threadIdx.x; i < p.rank; i += blockDim.x) st<TC>(dst, i, crow[i] * inv * p.cw[i]);
+            const float* kr = crow + p.rank;
+            for (int i = threadIdx.x; i < p.r; i += blockDim.x) st<TC>(dst, p.rank + i, rotated_elem(kr, i, p.rot, p.interleaved, cs, sn));
+        }
     }
     TC* qd = static_cast<TC*>(p.q_out) + (size_t)t * p.H * dq;
     for (int i = threadIdx.x; i < p.H * dq; i += blockDim.x) {
@@ -1544,10 +1517,13 @@ template <typename TO> __global__ void head_gate_kernel(TO* out, const float* in
 template <typename TO, int NW> __global__ __launch_bounds__(64 * NW) void moe_route_kernel(int32_t* ids, float* wts, float* sgate, TO* xn, const float* x,
                                                                                const float* norm_w, const float* router, const float* corr,
                                                                                const float* gate_row, int width, int E, int K, float scale,
-                                                                               float eps, int append) {
+                                                                               float eps, int append, int sig, int groups, int keep, int normalise) {
     extern __shared__ __align__(16) float rsm[];
     float* hs = rsm;                       // [width]
     float* logit = hs + width;             // [E + 1]
+    float* sc = logit + E + 1;             // [E] scores
+    float* cv = sc + E;                    // [E] choice scores
+    float* gs = cv + E;                    // [E] group scores
     __shared__ float red[NW];
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float* xr = x + (size_t)t * width;
@@ -1594,19 +1570,45 @@ template <typename TO, int NW> __global__ __launch_bounds__(64 * NW) void moe_ro
         if (sgate) sgate[t] = sg;
         if (append) { ids[(size_t)t * KS + K] = E; wts[(size_t)t * KS + K] = sg; }
     }
-    float m = -INFINITY;
-    for (int e = lane; e < E; e += 64) m = fmaxf(m, logit[e]);
-    m = wave_max(m);
-    float den = 0.f;
-    for (int e = lane; e < E; e += 64) den += expf(logit[e] - m);
-    den = wave_sum(den);
+    // scores s (softmax or sigmoid of the logits) and choice scores s + correction, in LDS
+    if (sig) {
+        for (int e = lane; e < E; e += 64) { const float v = sigmoidf_(logit[e]); sc[e] = v; cv[e] = v + (corr ? corr[e] : 0.f); }
+    } else {
+        float m = -INFINITY;
+        for (int e = lane; e < E; e += 64) m = fmaxf(m, logit[e]);
+        m = wave_max(m);
+        float den = 0.f;
+        for (int e = lane; e < E; e += 64) den += expf(logit[e] - m);
+        den = wave_sum(den);
+        for (int e = lane; e < E; e += 64) { const float v = expf(logit[e] - m) / den; sc[e] = v; cv[e] = v + (corr ? corr[e] : 0.f); }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier();
+    if (groups > 0) {
+        // a group's score: the sum of its two largest choice scores (its only one when a group is one expert); the experts of every
+        // group but the keep best (ties to the lower group) leave the choice
+        const int per = E / groups;
+        for (int g = lane; g < groups; g += 64) {
+            float b1 = -INFINITY, b2 = -INFINITY;
+            for (int i = 0; i < per; ++i) { const float v = cv[g * per + i]; if (v > b1) { b2 = b1; b1 = v; } else if (v > b2) b2 = v; }
+            gs[g] = per > 1 ? b1 + b2 : b1;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier();
+        for (int g = lane; g < groups; g += 64) {
+            const float mine = gs[g];
+            int rank = 0;
+            for (int o = 0; o < groups; ++o) rank += (gs[o] > mine || (gs[o] == mine && o < g)) ? 1 : 0;
+            if (rank >= keep) for (int i = 0; i < per; ++i) cv[g * per + i] = -INFINITY;
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront"); __builtin_amdgcn_wave_barrier();
+    }
     // lane owns experts lane, lane + 64, ...: K rounds of (my best untaken choice score) -> wave maximum -> the lowest expert that has it
     unsigned long long taken = 0ull;                                    // bit i: my expert lane + 64 i is chosen already
+    float wsum = 0.f;
     for (int j = 0; j < K; ++j) {
         float bv = -INFINITY; int be = 0x7fffffff;
         for (int e = lane, i = 0; e < E; e += 64, ++i) {
-            const float cv = expf(logit[e] - m) / den + (corr ? corr[e] : 0.f);
-            if (!((taken >> i) & 1ull) && (cv > bv || be == 0x7fffffff)) { bv = cv; be = e; }
+            const float c = cv[e];
+            if (!((taken >> i) & 1ull) && (c > bv || be == 0x7fffffff)) { bv = c; be = e; }
         }
         const float top = wave_max(bv);
         int cand = (be != 0x7fffffff && bv == top) ? be : 0x7fffffff;
@@ -1615,8 +1617,13 @@ template <typename TO, int NW> __global__ __launch_bounds__(64 * NW) void moe_ro
         if (lane == (cand & 63)) taken |= 1ull << (cand >> 6);
         if (lane == 0) {
             ids[(size_t)t * KS + j] = cand;
-            wts[(size_t)t * KS + j] = expf(logit[cand] - m) / den * scale;
+            wts[(size_t)t * KS + j] = sc[cand] * scale;
+            wsum += sc[cand];
         }
+    }
+    if (normalise && lane == 0) {
+        const float inv = 1.f / (wsum + 1e-20f);
+        for (int j = 0; j < K; ++j) wts[(size_t)t * KS + j] *= inv;
     }
 }
 
@@ -1727,8 +1734,6 @@ int g_attn_wider = 1;           // A/B: twelve waves per (token, head) for the s
 int g_attn_group = 1;           // 0: grouped-query prompt steps take the kernel with one wave per head (A/B, tests of both paths)
 int g_attn_mfma = 1;            // mi355_hyb_set_attention_mfma(0): prompt steps take the generic kernel too (A/B, tests of both paths)
 
-#define LAUNCH_OK() do { const hipError_t e_ = hipGetLastError(); if (e_ != hipSuccess) return (int)e_; } while (0)
-inline bool is_dt(int dt) { return dt == MI355_DTYPE_F32 || dt == MI355_DTYPE_BF16; }
 
 }  // namespace
 
@@ -1890,6 +1895,17 @@ int mi355_hyb_masked_attention(void* out, int32_t out_dtype, int32_t ldo, int32_
                                int32_t T, int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim, int32_t block_size,
                                int32_t max_blocks, int32_t window, int32_t keep_first, float scale, float out_scale, int32_t k_ld,
                                int32_t v_ld, float softcap, int32_t cross_values, int32_t dtype, int64_t stream) {
+    return mi355_hyb_biased_attention(out, out_dtype, ldo, out_off, q, k_pages, v_pages, block_tables, context_lens, cu_seqlens_q, tok_seq, sink,
+                                      nullptr, num_seqs, T, heads, kv_heads, dim, vdim, block_size, max_blocks, window, keep_first, scale,
+                                      out_scale, k_ld, v_ld, softcap, cross_values, dtype, stream);
+}
+
+int mi355_hyb_biased_attention(void* out, int32_t out_dtype, int32_t ldo, int32_t out_off, const void* q, const void* k_pages,
+                               const void* v_pages, const uint32_t* block_tables, const uint32_t* context_lens,
+                               const uint32_t* cu_seqlens_q, const int32_t* tok_seq, const float* sink, const float* dist,
+                               int32_t num_seqs, int32_t T, int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim,
+                               int32_t block_size, int32_t max_blocks, int32_t window, int32_t keep_first, float scale, float out_scale,
+                               int32_t k_ld, int32_t v_ld, float softcap, int32_t cross_values, int32_t dtype, int64_t stream) {
     if (keep_first < 0) return -1;
     if (!out || !q || !k_pages || !v_pages || !block_tables || !context_lens || !cu_seqlens_q || !tok_seq) return -1;
     if (!is_dt(dtype) || !is_dt(out_dtype) || heads <= 0 || kv_heads <= 0 || heads % kv_heads || dim <= 0 || vdim <= 0) return -1;
@@ -1909,6 +1925,7 @@ int mi355_hyb_masked_attention(void* out, int32_t out_dtype, int32_t ldo, int32_
                      k_ld % epv == 0 && v_ld % epv == 0;
     p.cpk = 64;
     p.keep = window > 0 ? keep_first : 0;
+    p.dist = dist;
     if (vec) { int c = 1; while (c < vdim / epv) c <<= 1; p.cp2 = c; c = 1; while (c < dim / epv) c <<= 1; p.cpk = c; }
     else if (vdim > 512) return -1;
     // prompt-sized steps over bf16 pages: the matrix-core kernel (a tile of 16 tokens never spans two sequences)
@@ -1986,11 +2003,17 @@ int mi355_hyb_conv_silu(float* out, const float* proj, int32_t ldp, int32_t off,
 int mi355_hyb_conv(float* out, const float* proj, int32_t ldp, int32_t off, const float* w, const float* conv_state,
                    int64_t state_stride, const uint32_t* context_lens, const uint32_t* cu_seqlens_q, const int32_t* state_slots,
                    const int32_t* tok_seq, int32_t num_seqs, int32_t T, int32_t channels, int32_t taps, int32_t act, int64_t stream) {
+    return mi355_hyb_conv_bias(out, proj, ldp, off, w, nullptr, conv_state, state_stride, context_lens, cu_seqlens_q, state_slots, tok_seq,
+                               num_seqs, T, channels, taps, act, stream);
+}
+int mi355_hyb_conv_bias(float* out, const float* proj, int32_t ldp, int32_t off, const float* w, const float* bias, const float* conv_state,
+                        int64_t state_stride, const uint32_t* context_lens, const uint32_t* cu_seqlens_q, const int32_t* state_slots,
+                        const int32_t* tok_seq, int32_t num_seqs, int32_t T, int32_t channels, int32_t taps, int32_t act, int64_t stream) {
     if (act != 0 && act != 1) return -1;
     if (!out || !proj || !w || !conv_state || !context_lens || !cu_seqlens_q || !state_slots || !tok_seq) return -1;
     if (channels <= 0 || taps < 1 || taps > 16) return -1;
     if (T <= 0) return 0;
-    ConvArgs p{out, proj, ldp, off, w, const_cast<float*>(conv_state), state_stride, context_lens, cu_seqlens_q, state_slots, tok_seq, channels, taps, T, act, 0, nullptr};
+    ConvArgs p{out, proj, ldp, off, w, const_cast<float*>(conv_state), state_stride, context_lens, cu_seqlens_q, state_slots, tok_seq, channels, taps, T, act, 0, nullptr, bias};
     const int64_t n = (int64_t)T * channels;
     conv_silu_kernel<<<(unsigned)((n + 255) / 256), 256, 0, to_stream(stream)>>>(p);
     LAUNCH_OK(); return 0;
@@ -2128,11 +2151,20 @@ int mi355_hyb_latent_prepare(void* q_out, void* pages, const float* proj, int32_
                              const float* c_norm_w, const float* cos_t, const float* sin_t, const int64_t* positions,
                              const int64_t* slot_mapping, int32_t T, int32_t heads, int32_t dim, int32_t rot_dim, int32_t kv_rank,
                              int32_t rot_dims, int32_t interleaved, float eps, int32_t dtype, int64_t stream) {
-    if (!q_out || !pages || !proj || !q_abs || !c_norm_w || !positions || !slot_mapping || !is_dt(dtype)) return -1;
+    if (!pages) return -1;
+    return mi355_hyb_latent_prepare_ex(q_out, pages, proj, ldp, q_off, proj, ldp, c_off, q_abs, c_norm_w, cos_t, sin_t, positions, slot_mapping, T,
+                                       heads, dim, rot_dim, kv_rank, rot_dims, interleaved, eps, dtype, stream);
+}
+int mi355_hyb_latent_prepare_ex(void* q_out, void* pages, const float* q_src, int32_t ldq, int32_t q_off, const float* c_src, int32_t ldc,
+                                int32_t c_off, const float* q_abs, const float* c_norm_w, const float* cos_t, const float* sin_t,
+                                const int64_t* positions, const int64_t* slot_mapping, int32_t T, int32_t heads, int32_t dim,
+                                int32_t rot_dim, int32_t kv_rank, int32_t rot_dims, int32_t interleaved, float eps, int32_t dtype,
+                                int64_t stream) {
+    if (!q_out || !q_src || !q_abs || !positions || !slot_mapping || !is_dt(dtype) || (pages && (!c_src || !c_norm_w))) return -1;
     if (heads <= 0 || dim <= 0 || rot_dim < 0 || kv_rank <= 0 || rot_dims < 0 || rot_dims > rot_dim || (rot_dims & 1)) return -1;
     if (rot_dims > 0 && (!cos_t || !sin_t)) return -1;
     if (T <= 0) return 0;
-    LatentPrepArgs p{q_out, pages, proj, ldp, q_off, c_off, q_abs, c_norm_w, cos_t, sin_t, positions, slot_mapping,
+    LatentPrepArgs p{q_out, pages, q_src, ldq, q_off, c_src, ldc, c_off, q_abs, c_norm_w, cos_t, sin_t, positions, slot_mapping,
                      heads, dim, rot_dim, kv_rank, rot_dims, interleaved ? 1 : 0, eps};
     if (dtype == MI355_DTYPE_F32) latent_prepare_kernel<float><<<T, 256, 0, to_stream(stream)>>>(p);
     else latent_prepare_kernel<uint16_t><<<T, 256, 0, to_stream(stream)>>>(p);
@@ -2179,15 +2211,24 @@ int mi355_hyb_scale_f32(float* x, float s, int64_t n, int64_t stream) {
 int mi355_hyb_moe_route(int32_t* expert_ids, float* weights, float* shared_gate, void* xn, int32_t out_dtype, const float* x,
                         const float* norm_w, const float* router, const float* correction, const float* gate_row, int32_t T,
                         int32_t width, int32_t experts, int32_t top, float scale, float eps, int32_t append_shared, int64_t stream) {
+    return mi355_hyb_moe_route_ex(expert_ids, weights, shared_gate, xn, out_dtype, x, norm_w, router, correction, gate_row, T, width, experts, top,
+                                  scale, eps, append_shared, 0, 0, 0, 0, stream);
+}
+int mi355_hyb_moe_route_ex(int32_t* expert_ids, float* weights, float* shared_gate, void* xn, int32_t out_dtype, const float* x,
+                           const float* norm_w, const float* router, const float* correction, const float* gate_row, int32_t T,
+                           int32_t width, int32_t experts, int32_t top, float scale, float eps, int32_t append_shared,
+                           int32_t sigmoid_scores, int32_t groups, int32_t keep_groups, int32_t normalise, int64_t stream) {
+    if (groups < 0 || (groups > 0 && (experts % groups || keep_groups < 1 || keep_groups > groups || (experts / groups) * keep_groups < top))) return -1;
     if (!expert_ids || !weights || !x || !router || width <= 0 || experts < 1 || experts > 4096 || top < 1 || top > experts) return -1;
     if ((gate_row && !shared_gate && !append_shared) || (append_shared && !gate_row) || (xn && !is_dt(out_dtype))) return -1;
     if (T <= 0) return 0;
-    const size_t lds = (size_t)(width + experts + 1) * sizeof(float);
+    const size_t lds = (size_t)(width + 4 * experts + 1) * sizeof(float);
     if (lds > 60000) return -1;
     // few tokens (decoding batches): sixteen waves per token, about one router row each; prompts: four
     const bool bf = xn && out_dtype == MI355_DTYPE_BF16;
 #define ROUTE(TO, NW) moe_route_kernel<TO, NW><<<T, 64 * NW, lds, to_stream(stream)>>>(expert_ids, weights, shared_gate, (TO*)xn, x, norm_w, router, \
-                                                                                       correction, gate_row, width, experts, top, scale, eps, append_shared ? 1 : 0)
+                                                                                       correction, gate_row, width, experts, top, scale, eps, append_shared ? 1 : 0, \
+                                                                                       sigmoid_scores ? 1 : 0, groups, keep_groups, normalise ? 1 : 0)
     if (T <= 256) { if (bf) ROUTE(uint16_t, 16); else ROUTE(float, 16); }
     else { if (bf) ROUTE(uint16_t, 4); else ROUTE(float, 4); }
 #undef ROUTE

@@ -54,7 +54,11 @@ struct HLayer {
     bool has_delta() const { return c.mixer == MI355_HYB_MIX_PARALLEL || c.mixer == MI355_HYB_MIX_DELTA; }
     bool is_latent() const { return c.mixer == MI355_HYB_MIX_LATENT; }
     bool is_conv_attn() const { return c.mixer == MI355_HYB_MIX_CONV_ATTENTION; }
+    bool is_ssd() const { return c.mixer == MI355_HYB_MIX_SSD; }
     bool uses_pages() const { return has_attn() || is_latent() || is_conv_attn(); }
+    bool owns_pages() const { return uses_pages() && !c.kv_from; }       // a layer with kv_from reads another layer's pages
+    int ssd_inner() const { return c.d_heads * c.d_vdim; }
+    int ssd_channels() const { return c.d_heads * c.d_vdim + 2 * c.d_kv_heads * c.d_dim; }   // x | B | C: what the convolution sees
     bool rotates() const { return (has_attn() || is_latent()) && c.a_rot_dims > 0; }
     int conv_channels() const { return 2 * c.d_kv_heads * c.d_dim + c.d_heads * c.d_vdim; }
     int a_conv_channels() const { return (c.a_heads + c.a_kv_heads) * c.a_dim + c.a_kv_heads * c.a_vdim; }
@@ -79,6 +83,12 @@ struct HModel {
     int32_t* tok_seq = nullptr;
     // residual form 2 / input convolution: what the sublayer's first product reads; mixture of experts: routing and the gathered rows
     void *pre = nullptr, *moe_act = nullptr;
+    // form 3 / depth average / token side input / query latent
+    float *y2 = nullptr, *hf = nullptr, *xs = nullptr, *side_g = nullptr;
+    void *side_a = nullptr, *cq = nullptr;
+    Weight side_table;
+    bool need_hf = false, need_xs = false;
+    int max_side = 0, max_q_rank = 0;
     float *moe_gu = nullptr, *moe_y = nullptr, *moe_wts = nullptr, *moe_sgate = nullptr;
     int32_t *moe_ids = nullptr, *moe_pos = nullptr, *moe_row_token = nullptr, *moe_table = nullptr;
     bool need_pre = false;
@@ -109,10 +119,16 @@ int in_proj_parts(const mi355_hybrid_layer& c, int32_t* off) {
         return 3 * c.g_width;
     }
     if (c.mixer == MI355_HYB_MIX_LATENT) {
-        off[P_AQ] = r; r += c.a_heads * (c.a_dim + c.a_rot_dim);
-        off[P_AK] = r; r += c.a_kv_rank + c.a_rot_dim;
-        if (c.a_head_gate) { off[P_G] = r; r += c.a_heads; }
+        off[P_AQ] = r; r += c.a_q_rank > 0 ? c.a_q_rank : c.a_heads * (c.a_dim + c.a_rot_dim);
+        if (!c.kv_from) { off[P_AK] = r; r += c.a_kv_rank + c.a_rot_dim; }
+        if (c.a_out_gate) { off[P_G] = r; r += c.a_heads * c.a_vdim; }
+        else if (c.a_head_gate) { off[P_G] = r; r += c.a_heads; }
         return r;
+    }
+    if (c.mixer == MI355_HYB_MIX_SSD) {                                  // [gate z | x | B | C | dt]
+        const int inner = c.d_heads * c.d_vdim, gn = c.d_kv_heads * c.d_dim;
+        off[P_G] = 0; off[P_DV] = inner; off[P_DK] = 2 * inner; off[P_DQ] = 2 * inner + gn; off[P_A] = 2 * inner + 2 * gn;
+        return 2 * inner + 2 * gn + c.d_heads;
     }
     if (c.mixer == MI355_HYB_MIX_PARALLEL || c.mixer == MI355_HYB_MIX_ATTENTION || c.mixer == MI355_HYB_MIX_CONV_ATTENTION) {
         off[P_AQ] = r; r += c.a_heads * c.a_dim;
@@ -133,7 +149,17 @@ int in_proj_parts(const mi355_hybrid_layer& c, int32_t* off) {
 bool layer_ok(const mi355_hybrid_layer& c) {
     const bool attn = c.mixer == MI355_HYB_MIX_PARALLEL || c.mixer == MI355_HYB_MIX_ATTENTION;
     const bool delta = c.mixer == MI355_HYB_MIX_PARALLEL || c.mixer == MI355_HYB_MIX_DELTA;
-    if (c.mixer < 0 || c.mixer > MI355_HYB_MIX_CONV_ATTENTION || c.share_with < 0) return false;
+    if (c.mixer < 0 || c.mixer > MI355_HYB_MIX_SSD || c.share_with < 0) return false;
+    if (c.mixer == MI355_HYB_MIX_SSD) {
+        if (c.d_heads <= 0 || c.d_kv_heads <= 0 || c.d_heads % c.d_kv_heads || c.d_dim <= 0 || c.d_dim > 256 || c.d_vdim <= 0) return false;
+        if (c.d_conv < 1 || c.d_conv > 16 || c.d_norm_groups < 1 || (c.d_heads * c.d_vdim) % c.d_norm_groups) return false;
+    }
+    if (c.a_q_rank < 0 || c.kv_from < 0 || c.side_dim < 0 || c.side_col < 0 || c.depth_terms < 0 || c.moe_groups < 0) return false;
+    if ((c.a_q_rank || c.a_out_gate || c.kv_from) && c.mixer != MI355_HYB_MIX_LATENT) return false;
+    if (c.a_out_gate && c.a_head_gate) return false;
+    if (c.a_dist_bias && c.mixer != MI355_HYB_MIX_CONV_ATTENTION) return false;
+    if (c.moe_groups > 0 && (c.mlp_kind != 3 || c.moe_experts % c.moe_groups || c.moe_keep_groups < 1 || c.moe_keep_groups > c.moe_groups ||
+                             (c.moe_experts / c.moe_groups) * c.moe_keep_groups < c.moe_top)) return false;
     if (c.mixer == MI355_HYB_MIX_LATENT) {
         if (c.a_heads <= 0 || c.a_dim <= 0 || c.a_vdim <= 0 || c.a_kv_rank <= 0 || c.a_rot_dim < 0 || c.a_window < 0) return false;
         if (c.a_rot_dims < 0 || c.a_rot_dims > c.a_rot_dim || (c.a_rot_dims & 1) || c.a_softcap < 0.f) return false;
@@ -155,7 +181,7 @@ bool layer_ok(const mi355_hybrid_layer& c) {
         if (c.d_gate != MI355_HYB_GATE_SIGMOID_LR && c.d_gate != MI355_HYB_GATE_SILU) return false;
     }
     if (c.mixer == MI355_HYB_MIX_MINGRU && c.g_width <= 0) return false;
-    if (c.mlp_kind < 0 || c.mlp_kind > 3 || (c.mlp_kind && c.mlp_ff <= 0)) return false;
+    if (c.mlp_kind < 0 || c.mlp_kind > 4 || (c.mlp_kind && c.mlp_ff <= 0)) return false;
     if (c.mlp_kind == 3 && (c.moe_experts < 1 || c.moe_experts > 4096 || c.moe_top < 1 || c.moe_top > c.moe_experts || c.moe_shared_ff < 0)) return false;
     if (c.a_keep_first < 0 || c.in_conv < 0 || c.in_conv > 16) return false;
     if ((c.a_keep_first || c.a_norm_after_rot || c.a_head_temp) && !attn) return false;      // switches of the plain attention branch
@@ -167,7 +193,8 @@ bool is_matrix(int which) {
     switch (which) {
         case MI355_HW_EMBED: case MI355_HW_HEAD: case MI355_HW_IN_PROJ: case MI355_HW_OUT_PROJ: case MI355_HW_D_A2: case MI355_HW_D_G2:
         case MI355_HW_MLP_GATE_UP: case MI355_HW_MLP_DOWN: case MI355_HW_L_UKT: case MI355_HW_L_UV:
-        case MI355_HW_MOE_GATE_UP: case MI355_HW_MOE_DOWN: return true;
+        case MI355_HW_MOE_GATE_UP: case MI355_HW_MOE_DOWN: case MI355_HW_L_UQ: case MI355_HW_SIDE_GATE: case MI355_HW_SIDE_PROJ:
+        case MI355_HW_SIDE_TABLE: return true;
         default: return false;
     }
 }
@@ -175,8 +202,10 @@ bool is_matrix(int which) {
 int64_t expected_elems(const HModel* m, int layer, int which) {
     const int W = m->cfg.width;
     if (layer < 0) {
-        if (which == MI355_HW_EMBED || which == MI355_HW_HEAD) return (int64_t)m->cfg.vocab * W;
+        if (which == MI355_HW_EMBED) return (int64_t)m->cfg.vocab * W;
+        if (which == MI355_HW_HEAD) return m->cfg.tie_head ? -1 : (int64_t)m->cfg.vocab * W;
         if (which == MI355_HW_FINAL_NORM) return W;
+        if (which == MI355_HW_SIDE_TABLE) return m->cfg.side_cols > 0 ? (int64_t)m->cfg.vocab * m->cfg.side_cols : -1;
         return -1;
     }
     const HLayer& L = m->layers[layer];
@@ -184,7 +213,15 @@ int64_t expected_elems(const HModel* m, int layer, int which) {
     if (c.share_with) return -1;                               // a layer that runs on another layer's weights holds none
     switch (which) {
         case MI355_HW_NORM1: return W;
-        case MI355_HW_NORM2: return c.mlp_kind ? W : -1;
+        case MI355_HW_NORM2: return c.mlp_kind && m->cfg.residual_form != 3 ? W : -1;
+        case MI355_HW_D_SKIP: return L.is_ssd() ? c.d_heads : -1;
+        case MI355_HW_CONV_BIAS: return L.is_ssd() ? L.ssd_channels() : -1;
+        case MI355_HW_A_DIST: return L.is_conv_attn() && c.a_dist_bias ? 2 * c.a_heads : -1;
+        case MI355_HW_L_QNORM: return L.is_latent() && c.a_q_rank ? c.a_q_rank : -1;
+        case MI355_HW_L_UQ: return L.is_latent() && c.a_q_rank ? (int64_t)c.a_heads * (c.a_dim + c.a_rot_dim) * c.a_q_rank : -1;
+        case MI355_HW_SIDE_GATE: case MI355_HW_SIDE_PROJ: return c.side_dim ? (int64_t)c.side_dim * W : -1;
+        case MI355_HW_SIDE_NORM: return c.side_dim ? W : -1;
+        case MI355_HW_DEPTH_W: return c.depth_terms ? c.depth_terms : -1;
         case MI355_HW_IN_PROJ: return (int64_t)L.in_rows * W;
         case MI355_HW_IN_BIAS: return L.in_rows;
         case MI355_HW_OUT_PROJ: return (int64_t)W * L.out_k;
@@ -205,14 +242,18 @@ int64_t expected_elems(const HModel* m, int layer, int which) {
         case MI355_HW_A_TALK: return L.is_conv_attn() && c.a_talk ? c.a_heads * c.a_heads : -1;
         case MI355_HW_L_UKT: return L.is_latent() ? (int64_t)c.a_heads * c.a_kv_rank * c.a_dim : -1;
         case MI355_HW_L_UV: return L.is_latent() ? (int64_t)c.a_heads * c.a_vdim * c.a_kv_rank : -1;
-        case MI355_HW_L_CNORM: return L.is_latent() ? c.a_kv_rank : -1;
-        case MI355_HW_D_CONV: return L.has_delta() ? (int64_t)L.conv_channels() * c.d_conv : -1;
-        case MI355_HW_D_A_LOG: return L.has_delta() ? c.d_heads : -1;
-        case MI355_HW_D_DT_BIAS: return L.has_delta() ? (c.d_decay_channels ? c.d_heads * c.d_dim : c.d_heads) : -1;
-        case MI355_HW_D_NORM: return L.has_delta() ? c.d_vdim : -1;
+        case MI355_HW_L_CNORM: return L.is_latent() && !c.kv_from ? c.a_kv_rank : -1;
+        case MI355_HW_D_CONV: if (L.is_ssd()) return (int64_t)L.ssd_channels() * c.d_conv;
+                              return L.has_delta() ? (int64_t)L.conv_channels() * c.d_conv : -1;
+        case MI355_HW_D_A_LOG: return L.has_delta() || L.is_ssd() ? c.d_heads : -1;
+        case MI355_HW_D_DT_BIAS: if (L.is_ssd()) return c.d_heads;
+                                 return L.has_delta() ? (c.d_decay_channels ? c.d_heads * c.d_dim : c.d_heads) : -1;
+        case MI355_HW_D_NORM: if (L.is_ssd()) return L.ssd_inner();
+                              return L.has_delta() ? c.d_vdim : -1;
         case MI355_HW_D_A2: return L.has_delta() && c.d_decay_channels ? (int64_t)c.d_heads * c.d_dim * c.d_a_rank : -1;
         case MI355_HW_D_G2: return L.has_delta() && c.d_gate == MI355_HYB_GATE_SIGMOID_LR ? (int64_t)c.d_heads * c.d_vdim * c.d_g_rank : -1;
         case MI355_HW_MLP_GATE_UP: if (c.mlp_kind == 3) return c.moe_shared_ff && !L.shared_merged() ? (int64_t)2 * c.moe_shared_ff * W : -1;
+                                   if (c.mlp_kind == 4) return (int64_t)c.mlp_ff * W;
                                    return c.mlp_kind ? (int64_t)2 * c.mlp_ff * W : -1;
         case MI355_HW_MLP_DOWN: if (c.mlp_kind == 3) return c.moe_shared_ff && !L.shared_merged() ? (int64_t)W * c.moe_shared_ff : -1;
                                 return c.mlp_kind ? (int64_t)W * c.mlp_ff : -1;
@@ -221,7 +262,8 @@ int64_t expected_elems(const HModel* m, int layer, int which) {
 }
 
 Weight* slot_of(HModel* m, int layer, int which) {
-    if (layer < 0) return which == MI355_HW_EMBED ? &m->embed : which == MI355_HW_FINAL_NORM ? &m->final_norm : which == MI355_HW_HEAD ? &m->head : nullptr;
+    if (layer < 0) return which == MI355_HW_EMBED ? &m->embed : which == MI355_HW_FINAL_NORM ? &m->final_norm : which == MI355_HW_HEAD ? &m->head :
+                          which == MI355_HW_SIDE_TABLE ? &m->side_table : nullptr;
     if (layer >= (int)m->layers.size() || which < MI355_HW_NORM1 || which >= MI355_HW_COUNT) return nullptr;
     return &m->layers[layer].w[which];
 }
@@ -271,6 +313,11 @@ int ensure_capacity(HModel* m, int T, int n_out) {
         HCHECK(grow(m->att, t * (size_t)m->max_att * m->esize()));
         HCHECK(grow(m->tok_seq, t * 4));
         if (m->need_pre) HCHECK(grow(m->pre, t * W * m->esize()));
+        if (m->cfg.residual_form == 3) HCHECK(grow(m->y2, t * W * 4));
+        if (m->need_hf) HCHECK(grow(m->hf, t * W * 4));
+        if (m->need_xs) HCHECK(grow(m->xs, (m->layers.size() + 1) * t * W * 4));
+        if (m->max_side) { HCHECK(grow(m->side_g, t * (size_t)m->max_side * 4)); HCHECK(grow(m->side_a, t * (size_t)m->max_side * m->esize())); }
+        if (m->max_q_rank) HCHECK(grow(m->cq, t * (size_t)m->max_q_rank * m->esize()));
         if (m->max_moe_experts) {
             const size_t pairs = t * m->max_moe_top, rows = pairs + (size_t)(m->max_moe_experts + 1) * MOE_MAX_BLOCK_ROWS;
             HCHECK(grow(m->moe_ids, pairs * 4));
@@ -319,12 +366,26 @@ void* mi355_hybrid_create(const mi355_hybrid_config* cfg, const mi355_hybrid_lay
             if (std::memcmp(&a, &b, sizeof(a)) != 0) return nullptr;
         }
     }
-    if (cfg->residual_form < 0 || cfg->residual_form > 2 || cfg->norm_groups < 0 || (cfg->norm_groups > 1 && cfg->width % cfg->norm_groups)) return nullptr;
+    if (cfg->embed_scale != 0.f && cfg->embed_scale != 1.f && cfg->residual_form < 2) return nullptr;     // forms 0 / 1 read a bf16 copy of x
+    if (cfg->norm_kind < 0 || cfg->norm_kind > 1 || (cfg->norm_kind == 1 && cfg->residual_form != 3) || cfg->side_cols < 0 || cfg->logit_softcap < 0.f) return nullptr;
+    for (int i = 0; i < cfg->n_layers; ++i) {
+        const mi355_hybrid_layer& c = layers[i];
+        if (c.side_dim && c.side_col + c.side_dim > cfg->side_cols) return nullptr;
+        if (c.depth_terms && c.depth_terms != i + 2) return nullptr;
+        if (c.mlp_kind == 4 && cfg->residual_form != 3) return nullptr;
+        if (cfg->residual_form == 3 && (c.in_conv || c.share_with || c.moe_shared_ff || c.mlp_kind == 1 || c.mlp_kind == 2)) return nullptr;
+        if (c.kv_from) {                                            // the lender: an earlier latent layer with pages of its own and the same row
+            if (c.kv_from > i) return nullptr;
+            const mi355_hybrid_layer& b = layers[c.kv_from - 1];
+            if (b.mixer != MI355_HYB_MIX_LATENT || b.kv_from || b.a_kv_rank != c.a_kv_rank || b.a_rot_dim != c.a_rot_dim) return nullptr;
+        }
+    }
+    if (cfg->residual_form < 0 || cfg->residual_form > 3 || cfg->norm_groups < 0 || (cfg->norm_groups > 1 && cfg->width % cfg->norm_groups)) return nullptr;
     for (int i = 0; i < cfg->n_layers; ++i)                        // the experts' outputs are combined in front of an output norm
-        if (layers[i].mlp_kind == 3 && (cfg->residual_form == 1 || cfg->width > 4096)) return nullptr;
+        if (layers[i].mlp_kind == 3 && (cfg->residual_form == 1 || (cfg->residual_form != 3 && cfg->width > 4096))) return nullptr;
     HModel* m = new HModel();
     m->cfg = *cfg;
-    m->need_pre = cfg->residual_form == 2;
+    m->need_pre = cfg->residual_form == 2 || cfg->residual_form == 3;
     m->layers.resize(cfg->n_layers);
     int64_t off = 0;
     for (int i = 0; i < cfg->n_layers; ++i) {
@@ -339,6 +400,21 @@ void* mi355_hybrid_create(const mi355_hybrid_config* cfg, const mi355_hybrid_lay
         m->max_in_rows = std::max(m->max_in_rows, L.in_rows);
         m->max_mix = std::max(m->max_mix, L.out_k);
         if (L.has_attn() || L.is_conv_attn()) m->max_q = std::max(m->max_q, c.a_heads * c.a_dim);
+        if (L.is_ssd()) {
+            L.out_k = L.ssd_inner();
+            m->max_mix = std::max(m->max_mix, L.out_k);
+            m->max_conv = std::max(m->max_conv, L.ssd_channels());
+            m->max_o = std::max(m->max_o, L.ssd_inner());
+            L.conv_off = off; off += (int64_t)L.ssd_channels() * (c.d_conv - 1);
+            L.state_off = off; off += (int64_t)c.d_heads * c.d_dim * c.d_vdim;
+        }
+        if (c.side_dim) m->max_side = std::max(m->max_side, c.side_dim);
+        if (c.depth_terms) m->need_xs = true;
+        if (c.mlp_kind == 3 && cfg->residual_form == 3 && cfg->dtype == MI355_DTYPE_BF16) m->need_hf = true;
+        if (L.is_latent() && c.a_q_rank) {
+            m->max_q_rank = std::max(m->max_q_rank, c.a_q_rank);
+            m->max_aux2 = std::max(m->max_aux2, c.a_heads * (c.a_dim + c.a_rot_dim));
+        }
         if (L.is_latent()) {
             m->max_q = std::max(m->max_q, c.a_heads * (c.a_kv_rank + c.a_rot_dim));
             m->max_aux1 = std::max(m->max_aux1, c.a_heads * c.a_kv_rank);
@@ -379,11 +455,11 @@ void mi355_hybrid_destroy(void* mp) {
     drop_graphs(m);
     for (HLayer& L : m->layers) {
         for (Weight& w : L.w) if (w.p) (void)hipFree(w.p);
-        for (void* p : {(void*)L.cos_t, (void*)L.sin_t, L.k_pages, L.v_pages}) if (p) (void)hipFree(p);
+        for (void* p : {(void*)L.cos_t, (void*)L.sin_t, L.owns_pages() ? L.k_pages : nullptr, L.owns_pages() ? L.v_pages : nullptr}) if (p) (void)hipFree(p);
     }
     for (void* p : {m->embed.p, m->final_norm.p, m->head.p, (void*)m->state, (void*)m->prep, (void*)m->x, (void*)m->proj, (void*)m->aux1, (void*)m->aux2,
                     (void*)m->conv, (void*)m->o, (void*)m->y, (void*)m->gu, m->xcopy, m->q, m->mix, m->act, m->xn, m->att, (void*)m->tok_seq,
-                    m->pre, m->moe_act, (void*)m->moe_gu, (void*)m->moe_y, (void*)m->moe_wts, (void*)m->moe_sgate, (void*)m->moe_ids,
+                    m->pre, m->moe_act, (void*)m->y2, (void*)m->hf, (void*)m->xs, (void*)m->side_g, m->side_a, m->cq, m->side_table.p, (void*)m->moe_gu, (void*)m->moe_y, (void*)m->moe_wts, (void*)m->moe_sgate, (void*)m->moe_ids,
                     (void*)m->moe_pos, (void*)m->moe_row_token, (void*)m->moe_table})
         if (p) (void)hipFree(p);
     delete m;
@@ -432,7 +508,7 @@ int64_t mi355_hybrid_cache_bytes(void* mp, int32_t num_blocks) {
     if (!m || num_blocks < 0) return -1;
     int64_t b = m->slot_floats * 4 * m->cfg.state_slots;
     for (const HLayer& L : m->layers)
-        if (L.uses_pages()) b += (int64_t)num_blocks * m->cfg.block_size * (L.k_row() + L.v_row()) * (int64_t)m->esize();
+        if (L.owns_pages()) b += (int64_t)num_blocks * m->cfg.block_size * (L.k_row() + L.v_row()) * (int64_t)m->esize();
     return b;
 }
 
@@ -442,7 +518,7 @@ int mi355_hybrid_alloc_cache(void* mp, int32_t num_blocks) {
     HHIP(hipDeviceSynchronize());
     drop_graphs(m);
     for (HLayer& L : m->layers) {
-        if (!L.uses_pages()) continue;
+        if (!L.owns_pages()) continue;
         const size_t rows = (size_t)num_blocks * m->cfg.block_size;
         HCHECK(grow(L.k_pages, rows * L.k_row() * m->esize()));
         HHIP(hipMemset(L.k_pages, 0, rows * L.k_row() * m->esize()));
@@ -451,6 +527,7 @@ int mi355_hybrid_alloc_cache(void* mp, int32_t num_blocks) {
             HHIP(hipMemset(L.v_pages, 0, rows * L.v_row() * m->esize()));
         }
     }
+    for (HLayer& L : m->layers) if (L.c.kv_from) L.k_pages = m->layers[L.c.kv_from - 1].k_pages;
     const size_t sb = (size_t)m->slot_floats * 4 * m->cfg.state_slots;
     HCHECK(grow(m->state, sb));
     HHIP(hipMemset(m->state, 0, sb));
@@ -465,7 +542,7 @@ static int forward_check(HModel* m, const uint32_t* tokens, const int64_t* posit
                          int32_t max_blocks, int32_t max_context_len, float* logits) {
     if (!m || !tokens || !positions || !slot_mapping || !block_tables || !context_lens || !cu_seqlens_q || !state_slots) return -1;
     if (num_seqs <= 0 || T <= 0 || n_out < 0 || (n_out > 0 && (!out_rows || !logits)) || max_blocks <= 0) return -1;
-    if (!m->state || !m->embed.p || !m->final_norm.p || !m->head.p) return -3;
+    if (!m->state || !m->embed.p || !m->final_norm.p || (!m->head.p && !m->cfg.tie_head) || (m->cfg.side_cols > 0 && !m->side_table.p)) return -3;
     if ((int64_t)max_blocks * m->cfg.block_size < max_context_len) return -4;
     for (const HLayer& L : m->layers) {
         const HLayer& WL = L.c.share_with ? m->layers[L.c.share_with - 1] : L;
@@ -473,7 +550,7 @@ static int forward_check(HModel* m, const uint32_t* tokens, const int64_t* posit
             const int need[] = {MI355_HW_NORM1, MI355_HW_IN_PROJ, MI355_HW_OUT_PROJ};
             for (int s : need) if (!L.w[s].p) return -3;
             for (int s = MI355_HW_NORM2; s < MI355_HW_COUNT; ++s)
-                if (s != MI355_HW_IN_BIAS && s != MI355_HW_MOE_CORRECTION && expected_elems(m, (int)(&L - m->layers.data()), s) > 0 && !L.w[s].p) return -3;
+                if (s != MI355_HW_IN_BIAS && s != MI355_HW_MOE_CORRECTION && s != MI355_HW_CONV_BIAS && expected_elems(m, (int)(&L - m->layers.data()), s) > 0 && !L.w[s].p) return -3;
         }
         if (L.uses_pages() && (!L.k_pages || (L.rotates() && WL.n_pos < max_context_len))) return -4;
     }
@@ -488,11 +565,17 @@ static int forward_enqueue(HModel* m, const uint32_t* tokens, const int64_t* pos
     const float eps = m->cfg.norm_eps;
     const bool bf = m->bf16();
     const bool sandwich = m->cfg.residual_form == 2;                // a norm in front of every sublayer: nothing reads a copy of x
-    void* xcopy = (bf && !sandwich) ? m->xcopy : nullptr;
-    void* xin = sandwich ? m->pre : (bf ? m->xcopy : (void*)m->x);  // what the sublayers' first product reads
+    const bool parallel = m->cfg.residual_form == 3;                // one norm per layer, both sublayers read it
+    void* xcopy = (bf && !sandwich && !parallel) ? m->xcopy : nullptr;
+    void* xin = (sandwich || parallel) ? m->pre : (bf ? m->xcopy : (void*)m->x);  // what the sublayers' first product reads
     const int xin_dt = bf ? MI355_DTYPE_BF16 : MI355_DTYPE_F32;
+    const int64_t TW = (int64_t)T * W;
     HCHECK(mi355_hyb_token_seq(m->tok_seq, cu_seqlens_q, num_seqs, stream));
-    HCHECK(mi355_hyb_embed(m->x, xcopy, m->embed.p, tokens, T, W, m->cfg.vocab, dt, stream));
+    if (m->cfg.embed_scale != 0.f && m->cfg.embed_scale != 1.f)
+        HCHECK(mi355_hyb_embed_scaled(m->x, m->embed.p, tokens, T, W, m->cfg.vocab, m->cfg.embed_scale, dt, stream));
+    else
+        HCHECK(mi355_hyb_embed(m->x, xcopy, m->embed.p, tokens, T, W, m->cfg.vocab, dt, stream));
+    if (m->need_xs) HCHECK(mi355_hyb_copy_f32(m->xs, m->x, TW, stream));         // X_0 of the depth average
     for (size_t li = 0; li < m->layers.size(); ++li) {
         HLayer& L = m->layers[li];
         const mi355_hybrid_layer& c = L.c;
@@ -523,6 +606,9 @@ static int forward_enqueue(HModel* m, const uint32_t* tokens, const int64_t* pos
             min_ = m->pre;
         } else if (sandwich) {
             HCHECK(mi355_hyb_pre_norm(m->pre, dt, m->x, f(MI355_HW_PRE_NORM1), T, W, eps, stream));
+        } else if (parallel) {                                         // (the router wants the norm's output in f32)
+            HCHECK(mi355_hyb_pre_norm_ex(m->pre, dt, (c.mlp_kind == 3 && bf) ? m->hf : nullptr, m->x, W, f(MI355_HW_NORM1), T, W, m->cfg.norm_kind,
+                                         eps, stream));
         }
         HCHECK(mi355_hyb_linear(m->proj, ldp, min_, xin_dt, W, WL.w[MI355_HW_IN_PROJ].p, f(MI355_HW_IN_BIAS), T, L.in_rows, W, dt, stream));
         int mix_col = 0;
@@ -543,18 +629,27 @@ static int forward_enqueue(HModel* m, const uint32_t* tokens, const int64_t* pos
             // absorbed form: q_abs[t, h] = W_uk,h^T q_h (one launch over the heads), attention over the latent rows themselves with
             // ONE shared key/value head (keys [latent | rotated part], values = the latent part of the same page row), then W_uv,h
             // on every head's latent-sized output, the head gate, and the output projection
+            // (queries through a latent: the q part of the projection is W_dq h; its RMS norm, then W_uq gives the heads' rows)
             const int R = c.a_kv_rank, dq = R + c.a_rot_dim, H = c.a_heads;
-            HCHECK(mi355_hyb_linear_batched(m->aux1, H * R, R, m->proj + L.off[P_AQ], MI355_DTYPE_F32, ldp, c.a_dim + c.a_rot_dim,
+            const float* qsrc = m->proj;
+            int ldq = ldp, q_off = L.off[P_AQ];
+            if (c.a_q_rank) {
+                HCHECK(mi355_hyb_pre_norm_ex(m->cq, dt, nullptr, m->proj + L.off[P_AQ], ldp, f(MI355_HW_L_QNORM), T, c.a_q_rank, 0, eps, stream));
+                ldq = H * (c.a_dim + c.a_rot_dim); q_off = 0; qsrc = m->aux2;
+                HCHECK(mi355_hyb_linear(m->aux2, ldq, m->cq, dt, c.a_q_rank, WL.w[MI355_HW_L_UQ].p, nullptr, T, ldq, c.a_q_rank, dt, stream));
+            }
+            HCHECK(mi355_hyb_linear_batched(m->aux1, H * R, R, qsrc + q_off, MI355_DTYPE_F32, ldq, c.a_dim + c.a_rot_dim,
                                             WL.w[MI355_HW_L_UKT].p, (int64_t)R * c.a_dim, T, R, c.a_dim, H, dt, stream));
-            HCHECK(mi355_hyb_latent_prepare(m->q, L.k_pages, m->proj, ldp, L.off[P_AQ], L.off[P_AK], m->aux1, f(MI355_HW_L_CNORM), WL.cos_t,
-                                            WL.sin_t, positions, slot_mapping, T, H, c.a_dim, c.a_rot_dim, R, c.a_rot_dims,
-                                            c.a_rot_interleaved, eps, dt, stream));
+            HCHECK(mi355_hyb_latent_prepare_ex(m->q, c.kv_from ? nullptr : L.k_pages, qsrc, ldq, q_off, m->proj, ldp, c.kv_from ? 0 : L.off[P_AK],
+                                               m->aux1, c.kv_from ? nullptr : f(MI355_HW_L_CNORM), WL.cos_t, WL.sin_t, positions, slot_mapping, T, H,
+                                               c.a_dim, c.a_rot_dim, R, c.a_rot_dims, c.a_rot_interleaved, eps, dt, stream));
             HCHECK(mi355_hyb_window_attention_ex(m->att, dt, H * R, 0, m->q, L.k_pages, L.k_pages, block_tables, context_lens, cu_seqlens_q,
                                                  m->tok_seq, c.a_has_sink ? f(MI355_HW_A_SINK) : nullptr, num_seqs, T, H, 1, dq, R,
                                                  m->cfg.block_size, max_blocks, c.a_window, c.a_scale, 1.f, dq, dq, c.a_softcap, 0, dt, stream));
             HCHECK(mi355_hyb_linear_batched(m->o, H * c.a_vdim, c.a_vdim, m->att, dt, H * R, R, WL.w[MI355_HW_L_UV].p,
                                             (int64_t)c.a_vdim * R, T, c.a_vdim, R, H, dt, stream));
-            if (c.a_head_gate) HCHECK(mi355_hyb_head_gate(m->mix, dt, m->o, m->proj + L.off[P_G], ldp, T, H, c.a_vdim, stream));
+            if (c.a_out_gate) HCHECK(mi355_hyb_elem_gate(m->mix, dt, m->o, m->proj + L.off[P_G], ldp, T, H * c.a_vdim, stream));
+            else if (c.a_head_gate) HCHECK(mi355_hyb_head_gate(m->mix, dt, m->o, m->proj + L.off[P_G], ldp, T, H, c.a_vdim, stream));
             else HCHECK(mi355_hyb_head_gate(m->mix, dt, m->o, nullptr, 0, T, H, c.a_vdim, stream));
         }
         if (L.is_conv_attn()) {
@@ -575,11 +670,25 @@ static int forward_enqueue(HModel* m, const uint32_t* tokens, const int64_t* pos
                                                      c.a_scale, 1.f, 0, 0, c.a_softcap, 1, dt, stream));
                 HCHECK(mi355_hyb_head_mix(m->mix, dt, m->o, f(MI355_HW_A_TALK), T, H, G, c.a_vdim, stream));
             } else {
-                HCHECK(mi355_hyb_window_attention_ex(m->mix, dt, L.out_k, 0, m->q, L.k_pages, L.v_pages, block_tables, context_lens,
-                                                     cu_seqlens_q, m->tok_seq, c.a_has_sink ? f(MI355_HW_A_SINK) : nullptr, num_seqs, T, H,
-                                                     G, c.a_dim, c.a_vdim, m->cfg.block_size, max_blocks, c.a_window, c.a_scale, 1.f, 0, 0,
-                                                     c.a_softcap, 0, dt, stream));
+                HCHECK(mi355_hyb_biased_attention(m->mix, dt, L.out_k, 0, m->q, L.k_pages, L.v_pages, block_tables, context_lens,
+                                                  cu_seqlens_q, m->tok_seq, c.a_has_sink ? f(MI355_HW_A_SINK) : nullptr,
+                                                  c.a_dist_bias ? f(MI355_HW_A_DIST) : nullptr, num_seqs, T, H, G, c.a_dim, c.a_vdim,
+                                                  m->cfg.block_size, max_blocks, c.a_window, 0, c.a_scale, 1.f, 0, 0, c.a_softcap, 0, dt, stream));
             }
+        }
+        if (L.is_ssd()) {
+            // x | B | C through the convolution (bias, silu), the scan over the state slot, then the gate, the group norm and W_o
+            const int C = L.ssd_channels();
+            float* conv_state = m->state + L.conv_off;
+            HCHECK(mi355_hyb_conv_bias(m->conv, m->proj, ldp, L.off[P_DV], f(MI355_HW_D_CONV), f(MI355_HW_CONV_BIAS), conv_state, m->slot_floats,
+                                       context_lens, cu_seqlens_q, state_slots, m->tok_seq, num_seqs, T, C, c.d_conv, 1, stream));
+            HCHECK(mi355_hyb_conv_state_update(conv_state, m->slot_floats, m->proj, ldp, L.off[P_DV], context_lens, cu_seqlens_q, state_slots,
+                                               num_seqs, C, c.d_conv, stream));
+            HCHECK(mi355_hyb_ssd_scan(m->o, m->state + L.state_off, m->slot_floats, m->conv, C, m->proj + L.off[P_A], ldp, f(MI355_HW_D_A_LOG),
+                                      f(MI355_HW_D_DT_BIAS), f(MI355_HW_D_SKIP), context_lens, cu_seqlens_q, state_slots, num_seqs, T, c.d_heads,
+                                      c.d_kv_heads, c.d_dim, c.d_vdim, stream));
+            HCHECK(mi355_hyb_gate_group_norm(m->mix, dt, m->o, m->proj + L.off[P_G], ldp, f(MI355_HW_D_NORM), T, L.ssd_inner(), c.d_norm_groups,
+                                             eps, stream));
         }
         if (L.has_delta()) {
             const int C = L.conv_channels();
@@ -617,6 +726,32 @@ static int forward_enqueue(HModel* m, const uint32_t* tokens, const int64_t* pos
             return mi355_hyb_norm_add(m->x, xcopy, m->y, W, f(norm_slot), T, W, eps, stream);
         };
         HCHECK(mi355_hyb_linear(m->y, W, m->mix, dt, L.out_k, WL.w[MI355_HW_OUT_PROJ].p, nullptr, T, W, L.out_k, dt, stream));
+        if (parallel) {
+            // x <- x + mixer(h) + ff(h): the feed-forward reads the same h (m->pre) the mixer's projections read
+            if (c.mlp_kind == 3) {
+                const int E = c.moe_experts, K = c.moe_top, ff = c.mlp_ff, pairs = T * K;
+                HCHECK(mi355_hyb_moe_route_ex(m->moe_ids, m->moe_wts, nullptr, nullptr, dt, bf ? m->hf : static_cast<const float*>(m->pre), nullptr,
+                                              f(MI355_HW_MOE_ROUTER), f(MI355_HW_MOE_CORRECTION), nullptr, T, W, E, K,
+                                              c.moe_scale != 0.f ? c.moe_scale : 1.f, eps, 0, c.moe_sigmoid, c.moe_groups, c.moe_keep_groups,
+                                              c.moe_normalise, stream));
+                const int bm = std::min(mi355_hyb_moe_block_rows(pairs, E, 2 * ff, W, dt), mi355_hyb_moe_block_rows(pairs, E, W, ff, dt));
+                const int nb = (pairs + bm - 1) / bm + E;
+                HCHECK(mi355_hyb_moe_group(m->moe_pos, m->moe_row_token, m->moe_table, m->moe_ids, pairs, K, E, bm, nb, stream));
+                HCHECK(mi355_hyb_linear_grouped(m->moe_gu, 2 * ff, xin, xin_dt, W, m->moe_row_token, WL.w[MI355_HW_MOE_GATE_UP].p, (int64_t)2 * ff * W,
+                                                m->moe_table, bm, nb, 2 * ff, W, dt, stream));
+                HCHECK(mi355_hyb_silu_glu(m->moe_act, dt, m->moe_gu, nb * bm, ff, m->moe_table, bm, stream));
+                HCHECK(mi355_hyb_linear_grouped(m->moe_y, W, m->moe_act, dt, ff, nullptr, WL.w[MI355_HW_MOE_DOWN].p, (int64_t)W * ff, m->moe_table, bm,
+                                                nb, W, ff, dt, stream));
+                HCHECK(mi355_hyb_moe_combine_add(m->x, m->y, m->moe_y, m->moe_pos, m->moe_wts, T, W, K, stream));
+            } else if (c.mlp_kind == 4) {
+                HCHECK(mi355_hyb_linear(m->gu, c.mlp_ff, xin, xin_dt, W, WL.w[MI355_HW_MLP_GATE_UP].p, nullptr, T, c.mlp_ff, W, dt, stream));
+                HCHECK(mi355_hyb_relu2(m->act, dt, m->gu, (int64_t)T * c.mlp_ff, stream));
+                HCHECK(mi355_hyb_linear(m->y2, W, m->act, dt, c.mlp_ff, WL.w[MI355_HW_MLP_DOWN].p, nullptr, T, W, c.mlp_ff, dt, stream));
+                HCHECK(mi355_hyb_add2(m->x, m->y, m->y2, TW, stream));
+            } else {
+                HCHECK(mi355_hyb_add2(m->x, m->y, nullptr, TW, stream));
+            }
+        } else {
         HCHECK(residual(MI355_HW_NORM1));
         if (c.mlp_kind == 3) {
             // mixture of experts: route (with the norm in front of it in form 2), group the (token, expert) pairs into whole blocks per
@@ -653,15 +788,31 @@ static int forward_enqueue(HModel* m, const uint32_t* tokens, const int64_t* pos
             HCHECK(mi355_hyb_linear(m->y, W, m->act, dt, c.mlp_ff, WL.w[MI355_HW_MLP_DOWN].p, nullptr, T, W, c.mlp_ff, dt, stream));
             HCHECK(residual(MI355_HW_NORM2));
         }
+        }
+        if (c.side_dim) {
+            // the token's own input to this layer: x <- x + RMSnorm(W_proj (gelu_tanh(W_gate x) * e)) w, e = the token's columns of the side table
+            HCHECK(mi355_hyb_linear(m->side_g, c.side_dim, m->x, MI355_DTYPE_F32, W, WL.w[MI355_HW_SIDE_GATE].p, nullptr, T, c.side_dim, W, dt, stream));
+            HCHECK(mi355_hyb_side_act(m->side_a, dt, m->side_g, m->side_table.p, m->cfg.side_cols, c.side_col, tokens, T, c.side_dim, m->cfg.vocab,
+                                      dt, stream));
+            HCHECK(mi355_hyb_linear(m->y, W, m->side_a, dt, c.side_dim, WL.w[MI355_HW_SIDE_PROJ].p, nullptr, T, W, c.side_dim, dt, stream));
+            HCHECK(mi355_hyb_norm_add(m->x, xcopy, m->y, W, f(MI355_HW_SIDE_NORM), T, W, eps, stream));
+        }
+        if (c.depth_terms) HCHECK(mi355_hyb_depth_average(m->x, m->xs, f(MI355_HW_DEPTH_W), c.depth_terms, TW, stream));
+        else if (m->need_xs) HCHECK(mi355_hyb_copy_f32(m->xs + (li + 1) * (size_t)TW, m->x, TW, stream));
         if (layer_trace)
             HHIP(hipMemcpyAsync(layer_trace + li * (size_t)T * W, m->x, (size_t)T * W * 4, hipMemcpyDeviceToDevice, reinterpret_cast<hipStream_t>(stream)));
     }
     if (n_out > 0) {
-        HCHECK(mi355_hyb_gather_group_norm(m->xn, dt, m->x, out_rows, static_cast<const float*>(m->final_norm.p), n_out, W,
-                                           m->cfg.norm_groups, eps, stream));
-        HCHECK(mi355_hyb_linear(logits, m->cfg.vocab, m->xn, dt, W, m->head.p, nullptr, n_out, m->cfg.vocab, W, dt, stream));
+        if (m->cfg.norm_kind == 1)
+            HCHECK(mi355_hyb_gather_norm_ex(m->xn, dt, m->x, out_rows, static_cast<const float*>(m->final_norm.p), n_out, W, 1, eps, stream));
+        else
+            HCHECK(mi355_hyb_gather_group_norm(m->xn, dt, m->x, out_rows, static_cast<const float*>(m->final_norm.p), n_out, W,
+                                               m->cfg.norm_groups, eps, stream));
+        HCHECK(mi355_hyb_linear(logits, m->cfg.vocab, m->xn, dt, W, m->cfg.tie_head ? m->embed.p : m->head.p, nullptr, n_out, m->cfg.vocab, W, dt,
+                                stream));
         if (m->cfg.logit_scale != 0.f && m->cfg.logit_scale != 1.f)
             HCHECK(mi355_hyb_scale_f32(logits, m->cfg.logit_scale, (int64_t)n_out * m->cfg.vocab, stream));
+        if (m->cfg.logit_softcap > 0.f) HCHECK(mi355_hyb_tanh_cap(logits, m->cfg.logit_softcap, (int64_t)n_out * m->cfg.vocab, stream));
     }
     return 0;
 }

@@ -16,14 +16,16 @@ import torch
 from ._lib import lib, HybridConfig, HybridLayer, RopeScaling
 
 DT_F32, DT_BF16 = 0, 2
-MIX_PARALLEL, MIX_MINGRU, MIX_DELTA, MIX_ATTENTION, MIX_LATENT, MIX_CONV_ATTENTION = 0, 1, 2, 3, 4, 5
+MIX_PARALLEL, MIX_MINGRU, MIX_DELTA, MIX_ATTENTION, MIX_LATENT, MIX_CONV_ATTENTION, MIX_SSD = 0, 1, 2, 3, 4, 5, 6
 GATE_SILU, GATE_SIGMOID_LR = 0, 1
 ROPE_DEFAULT, ROPE_LLAMA3, ROPE_YARN = 0, 2, 4
 (HW_EMBED, HW_FINAL_NORM, HW_HEAD, HW_NORM1, HW_NORM2, HW_IN_PROJ, HW_IN_BIAS, HW_OUT_PROJ, HW_A_QNORM, HW_A_KNORM, HW_A_SINK, HW_D_CONV,
  HW_D_A_LOG, HW_D_DT_BIAS, HW_D_NORM, HW_D_A2, HW_D_G2, HW_MLP_GATE_UP, HW_MLP_DOWN, HW_A_CONV, HW_A_TALK, HW_L_UKT, HW_L_UV,
  HW_L_CNORM, HW_PRE_NORM1, HW_PRE_NORM2, HW_IN_CONV, HW_A_TEMP, HW_MOE_ROUTER, HW_MOE_CORRECTION, HW_MOE_GATE_UP,
- HW_MOE_DOWN) = range(32)
-MLP_CLAMPED_GLU, MLP_GELU_GLU, MLP_MOE = 1, 2, 3
+ HW_MOE_DOWN, HW_D_SKIP, HW_CONV_BIAS, HW_A_DIST, HW_L_QNORM, HW_L_UQ, HW_SIDE_GATE, HW_SIDE_PROJ, HW_SIDE_NORM, HW_DEPTH_W,
+ HW_SIDE_TABLE) = range(42)
+MLP_CLAMPED_GLU, MLP_GELU_GLU, MLP_MOE, MLP_RELU2 = 1, 2, 3, 4
+NORM_RMS, NORM_LAYER = 0, 1
 
 # constants the Sogodra design fixes
 SOGODRA_GLU_ALPHA = 1.702          # y = g sigmoid(1.702 g) (u + 1)
@@ -336,7 +338,139 @@ class KerolornSpec:
         return L, slots, rope
 
 
-SPECS = {"Sogodra": SogodraSpec, "Vivazen": VivazenSpec, "Kerolorn": KerolornSpec}       # config.json `architecture` -> its reader
+class Ones:
+    """a slot entry: n ones (a convolution of one tap that the checkpoint leaves out)"""
+
+    def __init__(self, n):
+        self.n = int(n)
+
+    def bits(self, bits, shapes):
+        return np.full(self.n, 0x3F80, np.uint16)
+
+
+class SabolornSpec:
+    """config.json of a Sabolorn model -> layer structs + the tensor names behind every weight slot.  The design: ONE layer norm
+    (weight, no bias) per layer and both sublayers read it, x <- x + mixer(h) + ff(h); then the token's own input to the layer (a
+    slice of a second embedding table behind a gelu gate, RMS-normed), then a learned average over the embedding output and the
+    results of all layers so far.  Mixers: a state-space mixer with a scalar decay per head (`mamba2`), attention with biases, a short
+    convolution behind q / k / v and a logarithmic distance bias instead of a rotation (`attention`), latent attention with queries
+    through a latent of their own, yarn-scaled interleaved rotation and an elementwise output gate, optionally on the cached rows of
+    an earlier layer (`latent_attention`, `kv_from`).  Feed-forward: relu-squared dense or a mixture of experts with sigmoid scores,
+    group-limited choice and normalised weights.  Scaled embedding, tied output table, tanh-capped logits."""
+    residual_form, resid_alpha, norm_groups, norm_kind, tie_head = 3, 1.0, 1, NORM_LAYER, 1
+    rope_scaling = staticmethod(yarn_scaling)
+
+    def __init__(self, cfg, shapes):
+        if cfg.get("architecture") != "Sabolorn":
+            raise ValueError("not a Sabolorn config")
+        self.cfg = cfg
+        self.width, self.vocab = int(cfg["width"]), int(cfg["vocab"])
+        self.eps = float(cfg["norm"]["eps"])
+        self.embed_scale = float((cfg.get("embedding") or {}).get("scale", 1.0))
+        self.logit_softcap = float(cfg.get("logit_softcap") or 0.0)
+        side = cfg.get("token_side")
+        self.side_dim = int(side["dim"]) if side else 0
+        self.side_cols = int(shapes["side.embed"][1]) if side else 0
+        self.layers, self.slots, self.rope = [], [], []
+        for i, lc in enumerate(cfg["layers"]):
+            L, slots, rope = self._layer(i, "l%d." % i, lc, shapes)
+            self.layers.append(L)
+            self.slots.append(slots)
+            self.rope.append(rope)
+
+    def globals_(self):
+        """the tensors outside the layers: slot -> name"""
+        g = {HW_EMBED: "embed", HW_FINAL_NORM: "final.norm"}
+        if self.side_cols:
+            g[HW_SIDE_TABLE] = "side.embed"
+        return g
+
+    def _layer(self, i, p, lc, shapes):
+        L, slots, rope = HybridLayer(), {HW_NORM1: [p + "norm1"]}, None
+        c, kind, q = lc["mixer"], lc["type"], p + "mix."
+        if kind == "mamba2":
+            L.mixer = MIX_SSD
+            L.d_heads, L.d_vdim, L.d_dim, L.d_kv_heads = int(c["heads"]), int(c["vdim"]), int(c["state"]), int(c["groups"])
+            L.d_conv, L.d_norm_groups = int(c["conv"]), int(c.get("norm_groups", 1))
+            slots[HW_IN_PROJ], slots[HW_OUT_PROJ] = [q + "in"], [q + "o"]
+            slots[HW_D_CONV], slots[HW_CONV_BIAS] = [q + "conv"], [q + "conv.b"]
+            slots[HW_D_A_LOG], slots[HW_D_DT_BIAS], slots[HW_D_SKIP], slots[HW_D_NORM] = [q + "A_log"], [q + "dt_bias"], [q + "D"], [q + "norm"]
+        elif kind == "attention":
+            L.mixer = MIX_CONV_ATTENTION
+            L.a_heads, L.a_kv_heads, L.a_dim, L.a_vdim = int(c["heads"]), int(c["kv_heads"]), int(c["dim"]), int(c["vdim"])
+            L.a_scale, L.a_out_scale = float(c["scale"]), 1.0
+            slots[HW_IN_PROJ] = [q + "q", q + "k", q + "v"]
+            if q + "q.b" in shapes:
+                slots[HW_IN_BIAS] = [q + "q.b", q + "k.b", q + "v.b"]
+            if q + "q.conv" in shapes:
+                L.a_conv = int(shapes[q + "q.conv"][1])
+                slots[HW_A_CONV] = [q + "q.conv", q + "k.conv", q + "v.conv"]
+            else:
+                L.a_conv = 1
+                slots[HW_A_CONV] = [Ones((L.a_heads + L.a_kv_heads) * L.a_dim + L.a_kv_heads * L.a_vdim)]
+            if q + "r1" in shapes:
+                L.a_dist_bias = 1
+                slots[HW_A_DIST] = [q + "r1", q + "r2"]
+            slots[HW_OUT_PROJ] = [q + "o"]
+        elif kind == "latent_attention":
+            L.mixer = MIX_LATENT
+            L.a_heads, L.a_dim, L.a_vdim, L.a_scale, L.a_out_scale = int(c["heads"]), int(c["dim"]), int(c["vdim"]), float(c["scale"]), 1.0
+            L.a_kv_heads, L.a_kv_rank, L.a_rot_dim = 1, int(c["kv_rank"]), int(c["rot_dim"])
+            rope = c.get("rot")
+            L.a_rot_dims, L.a_rot_interleaved = (int(rope["dims"]) if rope else 0), 1
+            ins = []
+            if q + "dq" in shapes:
+                L.a_q_rank = int(shapes[q + "dq"][0])
+                ins.append(q + "dq")
+                slots[HW_L_QNORM], slots[HW_L_UQ] = [q + "dq.norm"], [q + "uq"]
+            else:
+                ins.append(q + "q")
+            if c.get("kv_from") is not None:
+                L.kv_from = int(c["kv_from"]) + 1
+            else:
+                ins.append(q + "dkv")
+                slots[HW_L_CNORM] = [q + "dkv.norm"]
+            if q + "g" in shapes:
+                ins.append(q + "g")
+                if int(shapes[q + "g"][0]) == L.a_heads * L.a_vdim:
+                    L.a_out_gate = 1
+                else:
+                    L.a_head_gate = 1
+            slots[HW_IN_PROJ], slots[HW_OUT_PROJ] = ins, [q + "o"]
+            slots[HW_L_UKT], slots[HW_L_UV] = [HeadTranspose(q + "uk", L.a_heads)], [q + "uv"]
+        else:
+            raise ValueError(f"layer type {kind!r} is not part of the design")
+        mlp = lc.get("mlp")
+        if mlp:
+            m = p + "mlp."
+            if mlp.get("kind") == "dense":
+                L.mlp_kind, L.mlp_ff = MLP_RELU2, int(mlp["ff"])
+                slots[HW_MLP_GATE_UP], slots[HW_MLP_DOWN] = [m + "up"], [m + "down"]
+            elif mlp.get("kind") == "moe":
+                r = mlp["router"]
+                L.mlp_kind, L.mlp_ff = MLP_MOE, int(mlp["expert"]["ff"])
+                L.moe_experts, L.moe_top, L.moe_scale = int(r["experts"]), int(r["top"]), 1.0
+                L.moe_sigmoid, L.moe_normalise = 1, 1
+                gr = r.get("groups")
+                if gr:
+                    L.moe_groups, L.moe_keep_groups = int(gr["count"]), int(gr["keep"])
+                slots[HW_MOE_ROUTER] = [m + "router"]
+                if m + "correction" in shapes:
+                    slots[HW_MOE_CORRECTION] = [m + "correction"]
+                slots[HW_MOE_GATE_UP] = [m + "e%d.%s" % (e, n) for e in range(L.moe_experts) for n in ("gate", "up")]
+                slots[HW_MOE_DOWN] = [m + "e%d.down" % e for e in range(L.moe_experts)]
+            else:
+                raise ValueError(f"feed-forward kind {mlp.get('kind')!r} is not part of the design")
+        if self.side_dim:
+            L.side_dim, L.side_col = self.side_dim, i * self.side_dim
+            slots[HW_SIDE_GATE], slots[HW_SIDE_PROJ], slots[HW_SIDE_NORM] = [p + "side.gate"], [p + "side.proj"], [p + "side.norm"]
+        if p + "dwa" in shapes:
+            L.depth_terms = int(shapes[p + "dwa"][0])
+            slots[HW_DEPTH_W] = [p + "dwa"]
+        return L, slots, rope
+
+
+SPECS = {"Sogodra": SogodraSpec, "Vivazen": VivazenSpec, "Kerolorn": KerolornSpec, "Sabolorn": SabolornSpec}       # config.json `architecture` -> its reader
 
 
 class HybridModel:
@@ -351,7 +485,9 @@ class HybridModel:
         c = HybridConfig(width=spec.width, vocab=spec.vocab, n_layers=n, dtype=self.dtype, block_size=self.block_size,
                          state_slots=self.state_slots, norm_eps=spec.eps, unit_eps=SOGODRA_UNIT_EPS,
                          residual_form=int(spec.residual_form), resid_alpha=float(spec.resid_alpha), norm_groups=int(spec.norm_groups),
-                         logit_scale=float(getattr(spec, "logit_scale", 1.0)))
+                         logit_scale=float(getattr(spec, "logit_scale", 1.0)), norm_kind=int(getattr(spec, "norm_kind", NORM_RMS)),
+                         embed_scale=float(getattr(spec, "embed_scale", 1.0)), logit_softcap=float(getattr(spec, "logit_softcap", 0.0)),
+                         tie_head=int(getattr(spec, "tie_head", 0)), side_cols=int(getattr(spec, "side_cols", 0)))
         self.h = lib.mi355_hybrid_create(ctypes.byref(c), self._layers)
         if not self.h:
             raise RuntimeError("mi355_hybrid_create refused the configuration")
@@ -383,7 +519,8 @@ class HybridModel:
         """bits: tensor name -> bf16 bits (uint16, any shape); shapes: name -> shape.  Concatenates what the host layer keeps as one
         matrix: the input projections along the rows, the output projections along k."""
         spec = self.spec
-        for which, name in ((HW_EMBED, "embed"), (HW_FINAL_NORM, "final.norm"), (HW_HEAD, "head")):
+        globals_ = spec.globals_() if hasattr(spec, "globals_") else {HW_EMBED: "embed", HW_FINAL_NORM: "final.norm", HW_HEAD: "head"}
+        for which, name in globals_.items():
             self._put(-1, which, bits[name])
         for i, slots in enumerate(spec.slots):
             for which, names in slots.items():
@@ -404,7 +541,7 @@ class HybridModel:
                     mats = [np.asarray(bits[nm], np.uint16).reshape(shapes[nm]) for nm in names]
                     self._put(i, which, np.concatenate(mats, axis=0))
                 else:
-                    self._put(i, which, np.concatenate([nm.bits(bits, shapes) if isinstance(nm, HeadTranspose)
+                    self._put(i, which, np.concatenate([nm.bits(bits, shapes) if isinstance(nm, (HeadTranspose, Ones))
                                                         else np.asarray(bits[nm], np.uint16).reshape(-1) for nm in names]))
 
     def load_state_dict_f32(self, W):

@@ -54,7 +54,7 @@ def _load_dense_llama(model_dir, config, dtype="bfloat16", **options):
     return load_dense_llama(model_dir, config, dtype=dtype, **options)
 
 
-for _name in ("Sogodra", "Vivazen", "Kerolorn"):
+for _name in ("Sogodra", "Vivazen", "Kerolorn", "Sabolorn"):
     register(_name, _load_layer_list, component="hybrid")
 for _name in ("LlamaForCausalLM", "MistralForCausalLM", "Qwen2ForCausalLM"):
     register(_name, _load_dense_llama)

@@ -32,6 +32,11 @@ extern "C" {
 #define MI355_HYB_MIX_CONV_ATTENTION 5 /* q, k, v pass a short causal convolution (a_conv taps, no activation), then attention with
                                       the a_* switches below; the convolution's last inputs live in the state slot */
 
+#define MI355_HYB_MIX_SSD 6         /* selective state-space mixer (scalar decay per head): the input projection gives [gate z | x | B | C |
+                                      step dt]; x, B, C pass a short causal convolution with bias and silu; per head S <- exp(-exp(a_log)
+                                      dt) S + dt B x^T, y = S^T C + skip x; y silu(z), RMS norm in d_norm_groups parts, output projection.
+                                      d_heads heads of d_vdim, state size d_dim, d_kv_heads groups of B / C, d_conv taps            */
+
 #define MI355_HYB_GATE_SILU 0      /* output gate silu(W_g h), full rank                */
 #define MI355_HYB_GATE_SIGMOID_LR 1 /* output gate sigmoid(W_g2 (W_g1 h)), low rank     */
 
@@ -85,6 +90,25 @@ typedef struct mi355_hybrid_layer {
      * renormalised).  moe_shared_ff > 0: one more expert of that size runs for every token, times sigmoid(w_sg . h)              */
     int32_t moe_experts, moe_top, moe_shared_ff;
     float moe_scale;
+    /* more switches of the router (all 0 = the form above) */
+    int32_t moe_sigmoid;           /* scores are sigmoid(z) instead of softmax(z)                                           */
+    int32_t moe_groups, moe_keep_groups; /* > 0: the experts form moe_groups equal groups of neighbours; a group's score is the sum of
+                                      its two largest choice scores and only experts of the best moe_keep_groups groups can be chosen */
+    int32_t moe_normalise;         /* the chosen experts' scores are divided by their sum (+ 1e-20) before moe_scale         */
+    /* feed-forward kind 4: dense without a gate, y = W_down relu(W_up h)^2 (MI355_HW_MLP_GATE_UP holds the [ff, width] up rows)  */
+    int32_t d_norm_groups;         /* MI355_HYB_MIX_SSD: parts of the gated output with a root mean square of their own      */
+    int32_t a_dist_bias;           /* MI355_HYB_MIX_CONV_ATTENTION: score <- score - r1[h] ln(1 + r2[h] (i - j)), MI355_HW_A_DIST */
+    int32_t a_q_rank;              /* latent attention, > 0: queries through a latent, q = W_uq RMSnorm(W_dq h) (MI355_HW_L_UQ,
+                                      MI355_HW_L_QNORM); the q part of the input projection then holds the a_q_rank rows of W_dq */
+    int32_t a_out_gate;            /* latent attention: the concatenated heads times sigmoid(W_g h) element by element, W_g
+                                      [heads vdim, width] in the gate part of the input projection                            */
+    int32_t kv_from;               /* latent attention, n > 0: no down-projection and no pages of its own; the layer reads the pages
+                                      that layer n - 1 (an earlier latent layer of the same kv_rank / rot_dim) has written       */
+    int32_t side_dim;              /* > 0: after the sublayers x <- x + RMSnorm(W_proj (gelu_tanh(W_gate x) * e)) w with e = the
+                                      token's row of the side table, columns [side_col, side_col + side_dim)                   */
+    int32_t side_col;
+    int32_t depth_terms;           /* n > 0: behind the layer x <- sum_j w[j] X_j over the n earliest of (embedding output, results
+                                      of the layers so far); n = layer index + 2 (MI355_HW_DEPTH_W [n])                        */
 } mi355_hybrid_layer;
 
 typedef struct mi355_hybrid_config {
@@ -101,6 +125,13 @@ typedef struct mi355_hybrid_config {
     int32_t norm_groups;           /* the layer norms and the last norm take the RMS over this many equal consecutive parts
                                       of the vector separately (0 or 1: over the whole vector)                       */
     float logit_scale;             /* the logits are multiplied by it (0 = 1)                                        */
+    /* residual_form 3: ONE norm per layer, h = norm(x) (MI355_HW_NORM1), and both sublayers read it: x <- x + mixer(h) + ff(h) */
+    int32_t norm_kind;             /* 0: RMS norm; 1: layer norm with a weight and no bias, (x - mean) / sqrt(var + eps) w -- the
+                                      norm in front of the sublayers (form 3) and the last norm                              */
+    float embed_scale;             /* the embedding rows are multiplied by it (0 = 1)                                        */
+    float logit_softcap;           /* > 0: logits <- cap tanh(logits / cap)                                                  */
+    int32_t tie_head;              /* the logits are taken against the embedding table itself; MI355_HW_HEAD stays empty     */
+    int32_t side_cols;             /* columns of the per-layer token table MI355_HW_SIDE_TABLE [vocab, side_cols] (0 = none) */
 } mi355_hybrid_config;
 
 /* weight slots: `layer` = -1 for the three global ones */
@@ -139,7 +170,17 @@ typedef struct mi355_hybrid_config {
                                       experts' size (moe_shared_ff == mlp_ff) is one more matrix at the end, here and in
                                       MOE_DOWN, and the dense slots stay empty                                       */
 #define MI355_HW_MOE_DOWN 31       /* [experts, width, ff]                                                           */
-#define MI355_HW_COUNT 32
+#define MI355_HW_D_SKIP 32         /* [heads]  state-space mixer: y += skip[h] x                                     */
+#define MI355_HW_CONV_BIAS 33      /* [channels] bias of the convolution MI355_HW_D_CONV                             */
+#define MI355_HW_A_DIST 34         /* [2, heads]: r1, then r2 of the distance bias                                   */
+#define MI355_HW_L_QNORM 35        /* [q_rank] weight of the query latent's RMS norm                                 */
+#define MI355_HW_L_UQ 36           /* [heads (dim + rot_dim), q_rank]                                                */
+#define MI355_HW_SIDE_GATE 37      /* [side_dim, width]                                                              */
+#define MI355_HW_SIDE_PROJ 38      /* [width, side_dim]                                                              */
+#define MI355_HW_SIDE_NORM 39      /* [width]                                                                        */
+#define MI355_HW_DEPTH_W 40        /* [depth_terms]                                                                  */
+#define MI355_HW_COUNT 41
+#define MI355_HW_SIDE_TABLE 41     /* global (layer -1): [vocab, side_cols]                                          */
 
 void* mi355_hybrid_create(const mi355_hybrid_config* cfg, const mi355_hybrid_layer* layers);
 void mi355_hybrid_destroy(void* model);
@@ -324,6 +365,72 @@ int mi355_hyb_moe_combine_norm_add(float* x, void* xcopy, const float* y_rows, c
                                    const float* y_shared, const float* shared_gate, const float* w, int32_t num_tokens, int32_t width,
                                    int32_t top, float eps, int64_t stream);
 int mi355_hyb_scale_f32(float* x, float s, int64_t n, int64_t stream);
+/* ---- mechanisms of the parallel-residual designs (hybrid_blocks.hip) */
+/* x f32 [T, width] = table rows ids times scale */
+int mi355_hyb_embed_scaled(float* x, const void* table, const uint32_t* ids, int32_t num_tokens, int32_t width, int32_t vocab, float scale,
+                           int32_t dtype, int64_t stream);
+/* out (dt_out) [T, width] (and out_f32, NULL or f32 [T, width]) = norm of the rows of x f32 [T, ldx] times w; kind 0: RMS, 1: layer
+ * norm (mean taken off, variance = mean of the squared deviations) */
+int mi355_hyb_pre_norm_ex(void* out, int32_t out_dtype, float* out_f32, const float* x, int32_t ldx, const float* w, int32_t num_tokens,
+                          int32_t width, int32_t kind, float eps, int64_t stream);
+/* mi355_hyb_gather_norm with the kind of norm as an argument */
+int mi355_hyb_gather_norm_ex(void* out, int32_t out_dtype, const float* x, const int32_t* rows, const float* w, int32_t n_rows,
+                             int32_t width, int32_t kind, float eps, int64_t stream);
+/* x f32 [T, width] += a + b (b NULL: += a) */
+int mi355_hyb_add2(float* x, const float* a, const float* b, int64_t n, int64_t stream);
+/* x[t] += y[t] + sum_j weights[t, j] y_rows[pos[t top + j]]  (y NULL = none): the experts' weighted sum without a norm */
+int mi355_hyb_moe_combine_add(float* x, const float* y, const float* y_rows, const int32_t* pos, const float* weights, int32_t num_tokens,
+                              int32_t width, int32_t top, int64_t stream);
+/* out (dt_out) [T, ff] = relu(u)^2 */
+int mi355_hyb_relu2(void* out, int32_t out_dtype, const float* u, int64_t n, int64_t stream);
+/* x <- cap tanh(x / cap) */
+int mi355_hyb_tanh_cap(float* x, float cap, int64_t n, int64_t stream);
+/* out (dt_out) [T, n] = in f32 [T, n] times sigmoid(gate_in[t, c]) element by element, gate_in f32 rows of ldg */
+int mi355_hyb_elem_gate(void* out, int32_t out_dtype, const float* in, const float* gate_in, int32_t ldg, int32_t num_tokens, int32_t n,
+                        int64_t stream);
+/* out (dt_out) [T, dim] = gelu_tanh(g[t, k]) * table (dt) [vocab, ldt] row ids[t], column col + k */
+int mi355_hyb_side_act(void* out, int32_t out_dtype, const float* g, const void* table, int32_t ldt, int32_t col, const uint32_t* ids,
+                       int32_t num_tokens, int32_t dim, int32_t vocab, int32_t dtype, int64_t stream);
+/* xs f32 [terms, n]: xs[terms - 1] <- x (the newest result), then x <- sum_j w[j] xs[j] */
+int mi355_hyb_depth_average(float* x, float* xs, const float* w, int32_t terms, int64_t n, int64_t stream);
+/* out (dt_out) [T, n] = (y * silu(gate_in[t, c])) / rms over each of `groups` equal parts * w[c]: the gate in front of the norm */
+int mi355_hyb_gate_group_norm(void* out, int32_t out_dtype, const float* y, const float* gate_in, int32_t ldg, const float* w,
+                              int32_t num_tokens, int32_t n, int32_t groups, float eps, int64_t stream);
+/* state-space scan over the new tokens of every sequence, state f32 [slots] x [heads, n_state, vdim] (stride in floats).
+ * xbc f32 [T, ldx]: x (heads x vdim) at 0, B (groups x n_state) behind it, C behind that, all behind the convolution and silu;
+ * dt_in f32 rows of ldd: the raw step per head; dt = softplus(dt_in + dt_bias[h]), decay = exp(-exp(a_log[h]) dt);
+ * S <- decay S + dt B x^T;  y f32 [T, heads, vdim] = S^T C + skip[h] x.  Head h reads group h / (heads / groups). */
+int mi355_hyb_ssd_scan(float* y, float* state, int64_t state_stride, const float* xbc, int32_t ldx, const float* dt_in, int32_t ldd,
+                       const float* a_log, const float* dt_bias, const float* skip, const uint32_t* context_lens,
+                       const uint32_t* cu_seqlens_q, const int32_t* state_slots, int32_t num_seqs, int32_t num_tokens, int32_t heads,
+                       int32_t groups, int32_t n_state, int32_t vdim, int64_t stream);
+/* mi355_hyb_conv with a bias per channel (NULL = none) in front of the activation */
+int mi355_hyb_conv_bias(float* out, const float* proj, int32_t ldp, int32_t off, const float* w, const float* bias, const float* conv_state,
+                        int64_t state_stride, const uint32_t* context_lens, const uint32_t* cu_seqlens_q, const int32_t* state_slots,
+                        const int32_t* token_seq, int32_t num_seqs, int32_t num_tokens, int32_t channels, int32_t taps, int32_t act,
+                        int64_t stream);
+/* mi355_hyb_masked_attention with a distance bias: dist f32 [2, heads] (NULL = none), score <- score - r1[h] ln(1 + r2[h] (i - j)) */
+int mi355_hyb_biased_attention(void* out, int32_t out_dtype, int32_t ldo, int32_t out_off, const void* q, const void* k_pages,
+                               const void* v_pages, const uint32_t* block_tables, const uint32_t* context_lens,
+                               const uint32_t* cu_seqlens_q, const int32_t* token_seq, const float* sink, const float* dist,
+                               int32_t num_seqs, int32_t num_tokens, int32_t heads, int32_t kv_heads, int32_t dim, int32_t vdim,
+                               int32_t block_size, int32_t max_blocks, int32_t window, int32_t keep_first, float scale, float out_scale,
+                               int32_t k_ld, int32_t v_ld, float softcap, int32_t cross_values, int32_t dtype, int64_t stream);
+/* mi355_hyb_latent_prepare with the query rows and the down-projection in buffers of their own: q_src f32 [T, ldq] holds per head
+ * [dim | rot_dim] at q_off; c_src f32 [T, ldc] holds [kv_rank | rot_dim] at c_off.  pages NULL: nothing is cached (a layer that reads
+ * another layer's pages) and c_src is not read */
+int mi355_hyb_latent_prepare_ex(void* q_out, void* pages, const float* q_src, int32_t ldq, int32_t q_off, const float* c_src, int32_t ldc,
+                                int32_t c_off, const float* q_abs, const float* c_norm_w, const float* cos_t, const float* sin_t,
+                                const int64_t* positions, const int64_t* slot_mapping, int32_t num_tokens, int32_t heads, int32_t dim,
+                                int32_t rot_dim, int32_t kv_rank, int32_t rot_dims, int32_t interleaved, float eps, int32_t dtype,
+                                int64_t stream);
+/* mi355_hyb_moe_route with the remaining switches: sigmoid_scores (s = sigmoid(z) instead of softmax), groups / keep_groups (> 0: only
+ * experts of the keep_groups groups with the largest sum of their two best choice scores can be chosen), normalise (weights divided
+ * by their sum + 1e-20 before the scale) */
+int mi355_hyb_moe_route_ex(int32_t* expert_ids, float* weights, float* shared_gate, void* xn, int32_t out_dtype, const float* x,
+                           const float* norm_w, const float* router, const float* correction, const float* gate_row, int32_t num_tokens,
+                           int32_t width, int32_t experts, int32_t top, float scale, float eps, int32_t append_shared,
+                           int32_t sigmoid_scores, int32_t groups, int32_t keep_groups, int32_t normalise, int64_t stream);
 /* 0: prompt-sized steps over bf16 pages take the generic kernel instead of the matrix-core ones; 2: the matrix-core kernel with one
  * wave per head also where the query heads of a key/value head could share a workgroup (A/B switch, process-wide; default 1) */
 void mi355_hyb_set_attention_mfma(int32_t on);
