@@ -187,10 +187,11 @@ def dense_ff(h, W, p):
     return np.maximum(h @ W[p + "up"].T, 0.0) ** 2 @ W[p + "down"].T
 
 
-def route(z, correction, top, groups=None):
+def route(z, correction, top, groups=None, margins=None):
     """z [T, E] router logits -> chosen experts [T, top] (largest choice score first, ties to the lower expert) and their weights:
     scores s = sigmoid(z); choice = s + correction; only experts of the groups[1] groups (of groups[0] equal groups of neighbours)
-    with the largest sum of their two best choice scores can be chosen; weights = s[chosen] / (their sum + 1e-20)"""
+    with the largest sum of their two best choice scores can be chosen; weights = s[chosen] / (their sum + 1e-20).
+    margins: a list that receives, per token, the smallest gap by which a group or an expert won its place"""
     E = z.shape[1]
     s = sigmoid(z)
     choice = s + correction if correction is not None else s.copy()
@@ -199,21 +200,27 @@ def route(z, correction, top, groups=None):
         per = E // cnt
         gs = np.sort(choice.reshape(-1, cnt, per), axis=-1)[:, :, -2:].sum(-1)
         order = np.argsort(-gs, axis=-1, kind="stable")[:, :keep]
+        if margins is not None and keep < cnt:
+            g2 = -np.sort(-gs, axis=-1)
+            margins.extend((g2[:, keep - 1] - g2[:, keep]).tolist())
         ok = np.zeros((z.shape[0], cnt), bool)
         np.put_along_axis(ok, order, True, axis=-1)
         choice = np.where(np.repeat(ok, per, axis=-1), choice, -np.inf)
     ids = np.argsort(-choice, axis=-1, kind="stable")[:, :top]
+    if margins is not None and top < E:
+        c2 = -np.sort(-choice, axis=-1)
+        margins.extend(np.where(np.isfinite(c2[:, top]), c2[:, top - 1] - c2[:, top], np.inf).tolist())
     w = np.take_along_axis(s, ids, axis=-1)
     return ids, w / (w.sum(-1, keepdims=True) + 1e-20)
 
 
-def moe_choice(h, W, p, r):
+def moe_choice(h, W, p, r, margins=None):
     gr = r.get("groups")
-    return route(h @ W[p + "router"].T, W.get(p + "correction"), r["top"], (gr["count"], gr["keep"]) if gr else None)
+    return route(h @ W[p + "router"].T, W.get(p + "correction"), r["top"], (gr["count"], gr["keep"]) if gr else None, margins)
 
 
-def moe_ff(h, W, p, m):
-    ids, w = moe_choice(h, W, p, m["router"])
+def moe_ff(h, W, p, m, margins=None):
+    ids, w = moe_choice(h, W, p, m["router"], margins)
     out = np.zeros((h.shape[0], W[p + "e0.down"].shape[0]))
     for t in range(h.shape[0]):
         for e, wt in zip(ids[t], w[t]):
@@ -228,8 +235,8 @@ def side_input(x, tokens, W, p, i, dim, eps):
     return x + rms_unit(y, eps) * W[p + "side.norm"]
 
 
-def forward(cfg, W, tokens):
-    """-> logits [T, vocab], the residual stream behind every layer [n_layers, T, width]"""
+def forward(cfg, W, tokens, margins=None):
+    """-> logits [T, vocab], the residual stream behind every layer [n_layers, T, width]; margins: see route()"""
     tokens = np.asarray(tokens, np.int64)
     eps = float(cfg["norm"]["eps"])
     x = W["embed"][tokens] * float(cfg["embedding"]["scale"])
@@ -252,7 +259,7 @@ def forward(cfg, W, tokens):
         m = lc.get("mlp")
         ff = 0.0
         if m:
-            ff = dense_ff(h, W, p + "mlp.") if m["kind"] == "dense" else moe_ff(h, W, p + "mlp.", m)
+            ff = dense_ff(h, W, p + "mlp.") if m["kind"] == "dense" else moe_ff(h, W, p + "mlp.", m, margins)
         x = x + (mix + ff)
         if cfg.get("token_side"):
             x = side_input(x, tokens, W, p, i, int(cfg["token_side"]["dim"]), eps)
@@ -285,7 +292,7 @@ def random_sabolorn(rng, cfg):
         W[name] = bf16_round(mean + s * rng.standard_normal(n))
 
     Wd, V, n_layers = cfg["width"], cfg["vocab"], len(cfg["layers"])
-    mat("embed", V, Wd, 1.0)
+    mat("embed", V, Wd, 0.25)                                             # also the output table: logits of a few units, below the cap
     vec("final.norm", Wd, 1.0)
     side = (cfg.get("token_side") or {}).get("dim", 0)
     if side:
