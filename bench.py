@@ -71,7 +71,7 @@ def parse():
     ap.add_argument("--hybrid", default="", metavar="SIZES",
                     help="instead of the default workload: the layer-list host layer (Sogodra design, random weights) beside the 16-bit llama "
                          "host layer at equal sizes -- comma list of 1b,3b,8b (bench_hybrid.py); prints its own JSON line")
-    ap.add_argument("--hybrid-design", default="sogodra", choices=["sogodra", "vivazen", "kerolorn"], help="--hybrid: which layer-list design")
+    ap.add_argument("--hybrid-design", default="sogodra", choices=["sogodra", "vivazen", "kerolorn", "sabolorn"], help="--hybrid: which layer-list design")
     ap.add_argument("--hybrid-prompt", type=int, default=2048, help="--hybrid: tokens of the prompt step")
     ap.add_argument("--hybrid-batch", type=int, default=8, help="--hybrid: sequences of the decode steps")
     ap.add_argument("--hybrid-ctx", type=int, default=2048, help="--hybrid: cached tokens behind every decoding sequence")

@@ -1,5 +1,5 @@
-"""`python bench.py --hybrid`: prompt and decode throughput of the layer-list host layer (Sogodra design, or Vivazen / Kerolorn with
-`--hybrid-design vivazen|kerolorn`; random weights) at layer sizes of a real model, beside the framework's closest existing model -- the 16-bit llama host layer (dense_model.cpp) -- at equal
+"""`python bench.py --hybrid`: prompt and decode throughput of the layer-list host layer (Sogodra design, or Vivazen / Kerolorn /
+Sabolorn with `--hybrid-design vivazen|kerolorn|sabolorn`; random weights) at layer sizes of a real model, beside the framework's closest existing model -- the 16-bit llama host layer (dense_model.cpp) -- at equal
 width, depth, head geometry, feed-forward size and vocabulary.  One GPU, bf16, synthetic data.  The default workload of bench.py and
 its one-line contract are not touched: this option prints its own JSON line.
 
@@ -35,6 +35,75 @@ KEROLORN = {
     "3b": dict(experts=16, top=3, keep=64, taps=4, layers=4),
     "8b": dict(experts=16, top=3, keep=64, taps=4, layers=4),
 }
+
+
+# Sabolorn at the same widths: a state-space layer (heads x 64, state 128, inner = 2 width), attention with the llama geometry behind
+# a convolution with a distance bias, latent attention with a query latent, and a second latent layer on the first one's pages; the
+# state-space layer has a relu^2 feed-forward of the llama size, the others a mixture of experts whose ACTIVE size equals it (`top`
+# experts of ff / 4 among 16 in 4 groups of which 2 stay open); a token side input of 256 columns per layer
+SABOLORN = {
+    "1b": dict(s_heads=64, s_vdim=64, s_state=128, s_groups=8, l_heads=16, l_dim=64, l_rot=64, l_rank=192, l_vdim=64, q_rank=768, taps=4,
+               experts=16, top=4, groups=4, keep=2, side=256, layers="mall"),
+    "3b": dict(s_heads=96, s_vdim=64, s_state=128, s_groups=8, l_heads=24, l_dim=64, l_rot=64, l_rank=192, l_vdim=64, q_rank=1024, taps=4,
+               experts=16, top=4, groups=4, keep=2, side=256, layers="mall"),
+    "8b": dict(s_heads=128, s_vdim=64, s_state=128, s_groups=8, l_heads=32, l_dim=128, l_rot=64, l_rank=192, l_vdim=128, q_rank=1536, taps=4,
+               experts=16, top=4, groups=4, keep=2, side=256, layers="mall"),
+}
+
+
+def sabolorn_config(s, v):
+    ssm = {"conv": v["taps"], "groups": v["s_groups"], "heads": v["s_heads"], "norm_groups": v["s_groups"], "state": v["s_state"], "vdim": v["s_vdim"]}
+    att = {"conv": v["taps"], "dim": s["dim"], "heads": s["heads"], "kv_heads": s["kv"], "scale": s["dim"] ** -0.5, "vdim": s["dim"]}
+    lat = {"dim": v["l_dim"], "heads": v["l_heads"], "kv_rank": v["l_rank"], "q_rank": v["q_rank"], "rot_dim": v["l_rot"], "vdim": v["l_vdim"],
+           "scale": (v["l_dim"] + v["l_rot"]) ** -0.5,
+           "rot": {"base": 10000.0, "dims": v["l_rot"], "scaling": {"factor": 8.0, "fast": 24.0, "original": 4096, "slow": 2.0}}}
+    moe = {"expert": {"ff": s["ff"] // 4}, "kind": "moe",
+           "router": {"experts": v["experts"], "groups": {"count": v["groups"], "keep": v["keep"]}, "top": v["top"]}}
+    dense = {"ff": s["ff"], "kind": "dense"}
+    layers, first = [], None
+    for i, c in enumerate(v["layers"]):
+        if c == "m":
+            layers.append({"type": "mamba2", "mixer": ssm, "mlp": dense})
+        elif c == "a":
+            layers.append({"type": "attention", "mixer": att, "mlp": moe})
+        else:
+            layers.append({"type": "latent_attention", "mixer": lat if first is None else dict(lat, kv_from=first), "mlp": moe})
+            first = i if first is None else first
+    return {"architecture": "Sabolorn", "embedding": {"scale": 0.5}, "layers": layers, "logit_softcap": 30.0, "norm": {"eps": 1e-5},
+            "token_side": {"dim": v["side"]}, "vocab": s["vocab"], "width": s["width"]}
+
+
+def sabolorn_shapes(cfg):
+    W, sh, n = cfg["width"], {}, len(cfg["layers"])
+    sh["embed"], sh["final.norm"], sh["side.embed"] = (cfg["vocab"], W), (W,), (cfg["vocab"], n * cfg["token_side"]["dim"])
+    for i, lc in enumerate(cfg["layers"]):
+        p, c, mlp = "l%d." % i, lc["mixer"], lc["mlp"]
+        q, m = p + "mix.", p + "mlp."
+        sh[p + "norm1"], sh[p + "dwa"] = (W,), (i + 2,)
+        sh[p + "side.gate"], sh[p + "side.proj"], sh[p + "side.norm"] = (cfg["token_side"]["dim"], W), (W, cfg["token_side"]["dim"]), (W,)
+        if lc["type"] == "mamba2":
+            inner, gn = c["heads"] * c["vdim"], c["groups"] * c["state"]
+            sh[q + "in"], sh[q + "conv"], sh[q + "conv.b"] = (2 * inner + 2 * gn + c["heads"], W), (inner + 2 * gn, c["conv"]), (inner + 2 * gn,)
+            sh[q + "dt_bias"], sh[q + "A_log"], sh[q + "D"], sh[q + "norm"], sh[q + "o"] = (c["heads"],), (c["heads"],), (c["heads"],), (inner,), (W, inner)
+        elif lc["type"] == "attention":
+            H, G, d, vd, t = c["heads"], c["kv_heads"], c["dim"], c["vdim"], c["conv"]
+            for nme, rows in (("q", H * d), ("k", G * d), ("v", G * vd)):
+                sh[q + nme], sh[q + nme + ".b"], sh[q + nme + ".conv"] = (rows, W), (rows,), (rows, t)
+            sh[q + "r1"], sh[q + "r2"], sh[q + "o"] = (H,), (H,), (W, H * vd)
+        else:
+            H, d, r, vd, rank, qr = c["heads"], c["dim"], c["rot_dim"], c["vdim"], c["kv_rank"], c["q_rank"]
+            sh[q + "dq"], sh[q + "dq.norm"], sh[q + "uq"] = (qr, W), (qr,), (H * (d + r), qr)
+            if "kv_from" not in c:
+                sh[q + "dkv"], sh[q + "dkv.norm"] = (rank + r, W), (rank,)
+            sh[q + "uk"], sh[q + "uv"], sh[q + "g"], sh[q + "o"] = (H * d, rank), (H * vd, rank), (H * vd, W), (W, H * vd)
+        if mlp and mlp["kind"] == "dense":
+            sh[m + "up"], sh[m + "down"] = (mlp["ff"], W), (W, mlp["ff"])
+        elif mlp:
+            ff, E = mlp["expert"]["ff"], mlp["router"]["experts"]
+            for e in range(E):
+                sh[m + "e%d.gate" % e], sh[m + "e%d.up" % e], sh[m + "e%d.down" % e] = (ff, W), (ff, W), (W, ff)
+            sh[m + "router"], sh[m + "correction"] = (E, W), (E,)
+    return sh
 
 
 def kerolorn_config(s, v):
@@ -156,7 +225,7 @@ def build_hybrid(cfg, max_tokens, slots):
     """random weights generated on the GPU, concatenated as the loader does it, handed over as device bf16"""
     import torch
     from candle_vllm_amd import hybrid_model as hm
-    shapes = {"Vivazen": vivazen_shapes, "Kerolorn": kerolorn_shapes, "Sogodra": sogodra_shapes}[cfg["architecture"]](cfg)
+    shapes = {"Vivazen": vivazen_shapes, "Kerolorn": kerolorn_shapes, "Sogodra": sogodra_shapes, "Sabolorn": sabolorn_shapes}[cfg["architecture"]](cfg)
     spec = hm.SPECS[cfg["architecture"]](cfg, shapes)
     m = hm.HybridModel(spec, dtype="bfloat16", block_size=64, state_slots=slots)
     g = torch.Generator(device="cuda").manual_seed(7)
@@ -171,7 +240,11 @@ def build_hybrid(cfg, max_tokens, slots):
         if name.endswith(".router"):
             return (2.0 * fan ** -0.5 * torch.randn(shape, generator=g, device="cuda")).to(torch.bfloat16)
         if name == "embed":
-            return torch.randn(shape, generator=g, device="cuda").to(torch.bfloat16)
+            return ((0.25 if cfg["architecture"] == "Sabolorn" else 1.0) * torch.randn(shape, generator=g, device="cuda")).to(torch.bfloat16)
+        if name.endswith(".r1") or name.endswith(".r2"):                  # the distance bias: positive rates
+            return (0.1 + torch.rand(shape, generator=g, device="cuda")).to(torch.bfloat16)
+        if name.endswith(".dwa"):
+            return torch.full(shape, 1.0 / shape[0], device="cuda").to(torch.bfloat16)
         if name.endswith(".talk"):
             return (torch.eye(shape[0], device="cuda") + 0.1 * torch.randn(shape, generator=g, device="cuda")).to(torch.bfloat16)
         s = 0.5 if name.endswith(".conv") else 0.3 if name.endswith("canon1") else (fan ** -0.5 if len(shape) > 1 else 0.3)
@@ -188,7 +261,8 @@ def build_hybrid(cfg, max_tokens, slots):
         nbytes += t.numel() * 2
         hm._check(hm.lib.mi355_hybrid_set_weight_dev(m.h, layer, which, t.data_ptr(), t.numel(), torch.cuda.current_stream().cuda_stream), "set_weight_dev")
         torch.cuda.synchronize()
-    for which, name in ((hm.HW_EMBED, "embed"), (hm.HW_FINAL_NORM, "final.norm"), (hm.HW_HEAD, "head")):
+    globals_ = spec.globals_() if hasattr(spec, "globals_") else {hm.HW_EMBED: "embed", hm.HW_FINAL_NORM: "final.norm", hm.HW_HEAD: "head"}
+    for which, name in globals_.items():
         put(-1, which, [name])
     for i, slots_ in enumerate(spec.slots):
         for which, names in slots_.items():
@@ -214,8 +288,9 @@ def run_size(name, T=2048, B=8, ctx=2048, dec_steps=16, design="sogodra"):
     from candle_vllm_amd.step_engine import StepEngine
     from oracle.dense_llama import DenseConfig
     s = SIZES[name]
-    extra = {"vivazen": VIVAZEN, "kerolorn": KEROLORN}.get(design, {}).get(name, {})
-    cfg = vivazen_config(s, extra) if design == "vivazen" else kerolorn_config(s, extra) if design == "kerolorn" else sogodra_config(s)
+    extra = {"vivazen": VIVAZEN, "kerolorn": KEROLORN, "sabolorn": SABOLORN}.get(design, {}).get(name, {})
+    cfg = (vivazen_config(s, extra) if design == "vivazen" else kerolorn_config(s, extra) if design == "kerolorn" else
+           sabolorn_config(s, extra) if design == "sabolorn" else sogodra_config(s))
     rng = np.random.default_rng(5)
     out = {"size": name, "design": design, "shape": dict(s, **extra), "prompt_tokens": T, "decode_batch": B,
            "decode_ctx": ctx}
@@ -286,8 +361,8 @@ def run_size(name, T=2048, B=8, ctx=2048, dec_steps=16, design="sogodra"):
 
 
 def main(sizes="1b,3b", prompt_tokens=2048, batch=8, ctx=2048, design="sogodra"):
-    if design not in ("sogodra", "vivazen", "kerolorn"):
-        raise SystemExit("--hybrid-design: sogodra, vivazen or kerolorn")
+    if design not in ("sogodra", "vivazen", "kerolorn", "sabolorn"):
+        raise SystemExit("--hybrid-design: sogodra, vivazen, kerolorn or sabolorn")
     res = [run_size(n.strip(), T=prompt_tokens, B=batch, ctx=ctx, design=design) for n in sizes.split(",") if n.strip()]
     print(json.dumps({"metric": "hybrid_vs_llama_throughput", "unit": "tokens/s", "dtype": "bf16", "data": "synthetic", "n_gpus": 1,
                       "note": "%s layer-list host layer beside the 16-bit llama host layer at equal sizes; the hybrid side's decode steps replay "

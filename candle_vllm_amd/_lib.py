@@ -431,6 +431,7 @@ _sig("mi355_hyb_tanh_cap", ctypes.c_int, [c_vp, c_f32, c_i64, c_i64])
 _sig("mi355_hyb_elem_gate", ctypes.c_int, [c_vp, c_i32, c_vp, c_vp, c_i32, c_i32, c_i32, c_i64])
 _sig("mi355_hyb_side_act", ctypes.c_int, [c_vp, c_i32, c_vp, c_vp, c_i32, c_i32, c_vp, c_i32, c_i32, c_i32, c_i32, c_i64])
 _sig("mi355_hyb_depth_average", ctypes.c_int, [c_vp, c_vp, c_vp, c_i32, c_i64, c_i64])
+_sig("mi355_hyb_layer_tail", ctypes.c_int, [c_vp, c_vp, c_vp, c_vp, c_vp, c_i32, c_vp, c_i32, c_vp, c_vp, c_i32, c_i32, c_i32, c_f32, c_i64])
 _sig("mi355_hyb_gate_group_norm", ctypes.c_int, [c_vp, c_i32, c_vp, c_vp, c_i32, c_vp, c_i32, c_i32, c_i32, c_f32, c_i64])
 _sig("mi355_hyb_ssd_scan", ctypes.c_int, [c_vp, c_vp, c_i64, c_vp, c_i32, c_vp, c_i32] + [c_vp] * 6 + [c_i32] * 6 + [c_i64])
 _sig("mi355_hyb_conv_bias", ctypes.c_int, [c_vp, c_vp, c_i32, c_i32, c_vp, c_vp, c_vp, c_i64, c_vp, c_vp, c_vp, c_vp] + [c_i32] * 5 + [c_i64])

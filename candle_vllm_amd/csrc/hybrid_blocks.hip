@@ -23,7 +23,7 @@ template <typename TW> __global__ void embed_scaled_kernel(float* x, const TW* t
 // One workgroup per row.  kind 0: x / sqrt(mean(x^2) + eps) w;  kind 1: (x - mean) / sqrt(mean((x - mean)^2) + eps) w (the mean is
 // taken off before the squares are summed: two passes over a row that stays in cache).  rows != NULL: row r of the output is row
 // rows[r] of x.
-template <typename TO> __global__ __launch_bounds__(256) void norm_rows_kernel(TO* out, float* out_f32, const float* x, int ldx, const int32_t* rows,
+template <typename TO> __global__ __launch_bounds__(1024) void norm_rows_kernel(TO* out, float* out_f32, const float* x, int ldx, const int32_t* rows,
                                                                              const float* w, int width, int kind, float eps) {
     __shared__ float red[16];
     const int r = blockIdx.x;
@@ -50,7 +50,7 @@ __global__ void add2_kernel(float* x, const float* a, const float* b, int64_t n)
 }
 
 // x[t] += y[t] + sum_j wts[t, j] rows[pos[t top + j]]; a workgroup per token, the token's rows and weights through LDS first
-__global__ __launch_bounds__(256) void moe_combine_add_kernel(float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ rows,
+__global__ __launch_bounds__(1024) void moe_combine_add_kernel(float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ rows,
                                                               const int32_t* __restrict__ pos, const float* __restrict__ wts, int width, int top) {
     extern __shared__ int csm[];
     int* sp = csm;
@@ -101,6 +101,49 @@ __global__ void depth_average_kernel(float* x, float* xs, const float* w, int te
     float acc = 0.f;
     for (int j = 0; j + 1 < terms; ++j) acc = fmaf(w[j], xs[(size_t)j * n + i], acc);
     x[i] = fmaf(w[terms - 1], cur, acc);
+}
+
+// The end of a layer and the start of the next in one launch, a workgroup per token row (a thread reads back only what it wrote):
+//   x += y / rms(y) * sw            (y != NULL: the token's side input)
+//   xs[terms - 1] <- x;  x <- sum_j dw[j] xs[j]      (dw != NULL: the average over the depth)
+//   out = norm(x) * nw              (nw != NULL: the norm the next layer's sublayers read; out_f32: a second copy in f32)
+template <typename TO> __global__ __launch_bounds__(1024) void layer_tail_kernel(float* x, const float* y, const float* sw, float* xs, const float* dw,
+                                                                               int terms, int64_t n, TO* out, float* out_f32, const float* nw, int width,
+                                                                               int kind, float eps) {
+    __shared__ float red[16];
+    const int t = blockIdx.x;
+    float* xr = x + (size_t)t * width;
+    float inv_y = 0.f;
+    if (y) {
+        const float* yr = y + (size_t)t * width;
+        float ss = 0.f;
+        for (int i = threadIdx.x; i < width; i += blockDim.x) ss = fmaf(yr[i], yr[i], ss);
+        inv_y = 1.f / sqrtf(block_sum(ss, red) / (float)width + eps);
+    }
+    float sum = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        float v = xr[i];
+        if (y) v += y[(size_t)t * width + i] * inv_y * sw[i];
+        if (dw) {
+            const size_t at = (size_t)t * width + i;
+            float acc = 0.f;
+            for (int j = 0; j + 1 < terms; ++j) acc = fmaf(dw[j], xs[(size_t)j * n + at], acc);
+            xs[(size_t)(terms - 1) * n + at] = v;
+            v = fmaf(dw[terms - 1], v, acc);
+        }
+        xr[i] = v;
+        sum += v;
+    }
+    if (!nw) return;
+    const float mean = kind == 1 ? block_sum(sum, red) / (float)width : 0.f;
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) { const float d = xr[i] - mean; ss = fmaf(d, d, ss); }
+    const float inv = 1.f / sqrtf(block_sum(ss, red) / (float)width + eps);
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        const float v = (xr[i] - mean) * inv * nw[i];
+        st<TO>(out, (size_t)t * width + i, v);
+        if (out_f32) out_f32[(size_t)t * width + i] = v;
+    }
 }
 
 // out = (y silu(z)) / rms over the part * w: a workgroup of 256 per (token, part)
@@ -228,8 +271,9 @@ int mi355_hyb_pre_norm_ex(void* out, int32_t out_dtype, float* out_f32, const fl
                           int32_t kind, float eps, int64_t stream) {
     if (!out || !x || !w || !is_dt(out_dtype) || width <= 0 || ldx < width || kind < 0 || kind > 1) return -1;
     if (T <= 0) return 0;
-    if (out_dtype == MI355_DTYPE_F32) norm_rows_kernel<float><<<T, 256, 0, to_stream(stream)>>>((float*)out, out_f32, x, ldx, nullptr, w, width, kind, eps);
-    else norm_rows_kernel<uint16_t><<<T, 256, 0, to_stream(stream)>>>((uint16_t*)out, out_f32, x, ldx, nullptr, w, width, kind, eps);
+    const int nt = (T <= 64 && width > 256) ? 1024 : 256;
+    if (out_dtype == MI355_DTYPE_F32) norm_rows_kernel<float><<<T, nt, 0, to_stream(stream)>>>((float*)out, out_f32, x, ldx, nullptr, w, width, kind, eps);
+    else norm_rows_kernel<uint16_t><<<T, nt, 0, to_stream(stream)>>>((uint16_t*)out, out_f32, x, ldx, nullptr, w, width, kind, eps);
     LAUNCH_OK(); return 0;
 }
 
@@ -253,7 +297,7 @@ int mi355_hyb_moe_combine_add(float* x, const float* y, const float* y_rows, con
                               int32_t top, int64_t stream) {
     if (!x || !y_rows || !pos || !weights || width <= 0 || top < 1 || top > 4096) return -1;
     if (T <= 0) return 0;
-    moe_combine_add_kernel<<<T, 256, (size_t)top * 8, to_stream(stream)>>>(x, y, y_rows, pos, weights, width, top);
+    moe_combine_add_kernel<<<T, (T <= 64 && width > 256) ? 1024 : 256, (size_t)top * 8, to_stream(stream)>>>(x, y, y_rows, pos, weights, width, top);
     LAUNCH_OK(); return 0;
 }
 
@@ -299,6 +343,20 @@ int mi355_hyb_depth_average(float* x, float* xs, const float* w, int32_t terms, 
     if (!x || !xs || !w || terms < 1) return -1;
     if (n <= 0) return 0;
     depth_average_kernel<<<blocks_of(n), 256, 0, to_stream(stream)>>>(x, xs, w, terms, n);
+    LAUNCH_OK(); return 0;
+}
+
+int mi355_hyb_layer_tail(float* x, const float* y, const float* side_w, float* xs, const float* depth_w, int32_t terms, void* out, int32_t out_dtype,
+                         float* out_f32, const float* norm_w, int32_t T, int32_t width, int32_t kind, float eps, int64_t stream) {
+    if (!x || width <= 0 || (y && !side_w) || (depth_w && (!xs || terms < 1)) || (norm_w && (!out || !is_dt(out_dtype))) || kind < 0 || kind > 1) return -1;
+    if (T <= 0) return 0;
+    const int64_t n = (int64_t)T * width;
+    // a row's passes are chains of loads: few rows (decoding batches) take 1024 threads a row so that a thread walks a quarter of the chain
+    const int nt = (T <= 64 && width > 256) ? 1024 : 256;
+    if (!norm_w || out_dtype == MI355_DTYPE_F32)
+        layer_tail_kernel<float><<<T, nt, 0, to_stream(stream)>>>(x, y, side_w, xs, depth_w, terms, n, (float*)out, out_f32, norm_w, width, kind, eps);
+    else
+        layer_tail_kernel<uint16_t><<<T, nt, 0, to_stream(stream)>>>(x, y, side_w, xs, depth_w, terms, n, (uint16_t*)out, out_f32, norm_w, width, kind, eps);
     LAUNCH_OK(); return 0;
 }
 

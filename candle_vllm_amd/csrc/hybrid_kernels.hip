@@ -491,7 +491,8 @@ struct AttnArgs {
     int keep;               // with a window: keys at positions < keep stay visible (the first tokens of the sequence)
     const float* dist;      // != NULL: [2, H] = r1, r2; score <- score - r1[h] ln(1 + r2[h] (query position - key position))
 };
-__device__ __forceinline__ float dist_bias(float r1, float r2, int d) { return r1 * log1pf(r2 * (float)d); }
+// (the hardware's log2: the argument is at least 1, so the absolute error stays near the f32 rounding of the score it is taken from)
+__device__ __forceinline__ float dist_bias(float r1, float r2, int d) { return r1 * 0.6931471805599453f * __log2f(fmaf(r2, (float)d, 1.f)); }
 __device__ __forceinline__ float cap_score(float s, float cap) { return cap > 0.f ? cap * tanhf(s / cap) : s; }
 // 16 bytes of a page row as floats (EPV = 8 bf16 or 4 f32)
 template <typename TC> struct Vec16;

@@ -606,7 +606,8 @@ static int forward_enqueue(HModel* m, const uint32_t* tokens, const int64_t* pos
             min_ = m->pre;
         } else if (sandwich) {
             HCHECK(mi355_hyb_pre_norm(m->pre, dt, m->x, f(MI355_HW_PRE_NORM1), T, W, eps, stream));
-        } else if (parallel) {                                         // (the router wants the norm's output in f32)
+        } else if (parallel && li == 0) {                              // (the router wants the norm's output in f32; the later layers'
+                                                                       //  norms are made at the end of the layer before them)
             HCHECK(mi355_hyb_pre_norm_ex(m->pre, dt, (c.mlp_kind == 3 && bf) ? m->hf : nullptr, m->x, W, f(MI355_HW_NORM1), T, W, m->cfg.norm_kind,
                                          eps, stream));
         }
@@ -795,10 +796,22 @@ static int forward_enqueue(HModel* m, const uint32_t* tokens, const int64_t* pos
             HCHECK(mi355_hyb_side_act(m->side_a, dt, m->side_g, m->side_table.p, m->cfg.side_cols, c.side_col, tokens, T, c.side_dim, m->cfg.vocab,
                                       dt, stream));
             HCHECK(mi355_hyb_linear(m->y, W, m->side_a, dt, c.side_dim, WL.w[MI355_HW_SIDE_PROJ].p, nullptr, T, W, c.side_dim, dt, stream));
-            HCHECK(mi355_hyb_norm_add(m->x, xcopy, m->y, W, f(MI355_HW_SIDE_NORM), T, W, eps, stream));
+            if (!parallel) HCHECK(mi355_hyb_norm_add(m->x, xcopy, m->y, W, f(MI355_HW_SIDE_NORM), T, W, eps, stream));
         }
-        if (c.depth_terms) HCHECK(mi355_hyb_depth_average(m->x, m->xs, f(MI355_HW_DEPTH_W), c.depth_terms, TW, stream));
-        else if (m->need_xs) HCHECK(mi355_hyb_copy_f32(m->xs + (li + 1) * (size_t)TW, m->x, TW, stream));
+        if (parallel) {
+            // the side input's norm and sum, the average over the depth and the norm that the next layer reads, in one launch
+            const bool more = li + 1 < m->layers.size();
+            const mi355_hybrid_layer* nx = more ? &m->layers[li + 1].c : nullptr;
+            HCHECK(mi355_hyb_layer_tail(m->x, c.side_dim ? m->y : nullptr, c.side_dim ? f(MI355_HW_SIDE_NORM) : nullptr, m->xs,
+                                        c.depth_terms ? f(MI355_HW_DEPTH_W) : nullptr, c.depth_terms, m->pre, dt,
+                                        (more && nx->mlp_kind == 3 && bf) ? m->hf : nullptr,
+                                        more ? static_cast<const float*>(m->layers[li + 1].w[MI355_HW_NORM1].p) : nullptr, T, W, m->cfg.norm_kind, eps,
+                                        stream));
+            if (!c.depth_terms && m->need_xs) HCHECK(mi355_hyb_copy_f32(m->xs + (li + 1) * (size_t)TW, m->x, TW, stream));
+        } else {
+            if (c.depth_terms) HCHECK(mi355_hyb_depth_average(m->x, m->xs, f(MI355_HW_DEPTH_W), c.depth_terms, TW, stream));
+            else if (m->need_xs) HCHECK(mi355_hyb_copy_f32(m->xs + (li + 1) * (size_t)TW, m->x, TW, stream));
+        }
         if (layer_trace)
             HHIP(hipMemcpyAsync(layer_trace + li * (size_t)T * W, m->x, (size_t)T * W * 4, hipMemcpyDeviceToDevice, reinterpret_cast<hipStream_t>(stream)));
     }

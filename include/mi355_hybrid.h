@@ -393,6 +393,11 @@ int mi355_hyb_side_act(void* out, int32_t out_dtype, const float* g, const void*
                        int32_t num_tokens, int32_t dim, int32_t vocab, int32_t dtype, int64_t stream);
 /* xs f32 [terms, n]: xs[terms - 1] <- x (the newest result), then x <- sum_j w[j] xs[j] */
 int mi355_hyb_depth_average(float* x, float* xs, const float* w, int32_t terms, int64_t n, int64_t stream);
+/* the end of a layer and the start of the next in one launch: x += y / rms(y) * side_w (y NULL: nothing added); then, with depth_w,
+ * mi355_hyb_depth_average over xs; then, with norm_w, out (dt_out) [T, width] (and out_f32, NULL or f32) = the norm of kind `kind` of
+ * the new x times norm_w (what mi355_hyb_pre_norm_ex would give) */
+int mi355_hyb_layer_tail(float* x, const float* y, const float* side_w, float* xs, const float* depth_w, int32_t terms, void* out, int32_t out_dtype,
+                         float* out_f32, const float* norm_w, int32_t num_tokens, int32_t width, int32_t kind, float eps, int64_t stream);
 /* out (dt_out) [T, n] = (y * silu(gate_in[t, c])) / rms over each of `groups` equal parts * w[c]: the gate in front of the norm */
 int mi355_hyb_gate_group_norm(void* out, int32_t out_dtype, const float* y, const float* gate_in, int32_t ldg, const float* w,
                               int32_t num_tokens, int32_t n, int32_t groups, float eps, int64_t stream);

@@ -312,6 +312,33 @@ def test_small_glue(lib, dtype):
     assert np.abs(x.cpu().numpy() - emb[tok] * 0.375).max() < 1e-6
 
 
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("T,W,terms,side,norm", [(5, 64, 3, True, True), (3, 50, 1, False, True), (2, 1100, 4, True, False), (4, 32, 0, True, True),
+                                                 (1, 8, 0, False, True)])
+def test_layer_tail_in_one_launch(lib, dtype, T, W, terms, side, norm):
+    """the side input's norm and sum, the average over the depth and the next layer's norm in one launch equal the three steps alone,
+    with any of them absent"""
+    _gpu()
+    rng = np.random.default_rng(T * W + terms)
+    x, y, sw, nw = f32(5 + rng.standard_normal((T, W))), f32(3 * rng.standard_normal((T, W))), f32(rng.standard_normal(W)), f32(1 + 0.2 * rng.standard_normal(W))
+    xs, dw = f32(rng.standard_normal((max(terms, 1), T * W))), f32(rng.uniform(0.1, 1, max(terms, 1)))
+    want_x = x + S.rms_unit(y, 1e-5) * sw if side else x.copy()
+    want_xs = xs.copy()
+    if terms:
+        want_xs[terms - 1] = want_x.reshape(-1)
+        want_x = (dw[:, None] * want_xs[:terms]).sum(0).reshape(T, W)
+    xd, xsd = dev(x), dev(xs)
+    out, out2 = empty_dt((T, W), dtype), torch.zeros((T, W), device="cuda")
+    ok(lib.mi355_hyb_layer_tail(xd.data_ptr(), P(y) if side else None, P(sw) if side else None, xsd.data_ptr(), P(dw) if terms else None, terms,
+                                out.data_ptr(), dtype, out2.data_ptr(), P(nw) if norm else None, T, W, 1, 1e-5, _st()))
+    assert np.abs(xd.cpu().numpy() - want_x).max() < 1e-5 * np.abs(want_x).max()
+    assert np.abs(xsd.cpu().numpy() - want_xs).max() < 1e-5 * max(1.0, np.abs(want_xs).max())
+    if norm:
+        h = S.layer_norm(want_x, nw, 1e-5)
+        assert np.abs(out2.cpu().numpy() - h).max() < 1e-4 * max(1.0, np.abs(h).max())
+        assert np.abs(host_dt(out, dtype) - h).max() < tol(dtype, 1e-4) * max(1.0, np.abs(h).max())
+
+
 # ------------------------------------------------------------------------------------------------------------ whole models
 def _moe(E, top, ff, groups=None):
     r = {"experts": E, "top": top}
