@@ -230,19 +230,22 @@ template <int DP, int LPC, int CH> __global__ __launch_bounds__(256) void ssd_sc
         const bool more = t0 + CH < te;
         if (more) fetch(t0 + CH);
         const int cn = min(CH, te - t0);
+        auto token = [&](int c) {
+            const float dec = sdec[buf][c], dx = sdt[buf][c] * vc[c];
+            float o = 0.f;
 #pragma unroll
-        for (int c = 0; c < CH; ++c) {
-            if (c < cn) {
-                const float dec = sdec[buf][c], dx = sdt[buf][c] * vc[c];
-                float o = 0.f;
-#pragma unroll
-                for (int r = 0; r < DP; ++r) {
-                    S[r] = fmaf(dec, S[r], dx * sB[buf][c][part][r]);
-                    o = fmaf(S[r], sC[buf][c][part][r], o);
-                }
-                o = column_sum<LPC>(o);
-                if (own && part == 0) p.y[((size_t)(t0 + c) * p.H + h) * vd + col] = fmaf(skip, vc[c], o);
+            for (int r = 0; r < DP; ++r) {
+                S[r] = fmaf(dec, S[r], dx * sB[buf][c][part][r]);
+                o = fmaf(S[r], sC[buf][c][part][r], o);
             }
+            o = column_sum<LPC>(o);
+            if (own && part == 0) p.y[((size_t)(t0 + c) * p.H + h) * vd + col] = fmaf(skip, vc[c], o);
+        };
+        if (cn == CH) {                                          // a whole chunk: no branch between the tokens, their LDS reads run ahead
+#pragma unroll
+            for (int c = 0; c < CH; ++c) token(c);
+        } else {
+            for (int c = 0; c < cn; ++c) token(c);
         }
         if (more) stage(buf ^ 1);
         __syncthreads();
@@ -387,8 +390,10 @@ int mi355_hyb_ssd_scan(float* y, float* state, int64_t state_stride, const float
         else ssd_scan_kernel<16, 4, 8><<<grid, 256, 0, s_>>>(p);
     } else {
         const dim3 grid(num_seqs, heads, (vdim + 15) / 16);
-        if (n_state <= 64) ssd_scan_kernel<4, 16, 8><<<grid, 256, 0, s_>>>(p);
-        else if (n_state <= 128) ssd_scan_kernel<8, 16, 8><<<grid, 256, 0, s_>>>(p);
+        // portions of prompts: 16 tokens per stage (the wait for a stage's rows is paid half as often); decoding batches: 8
+        const bool longer = num_tokens > 8 * num_seqs;
+        if (n_state <= 64) { if (longer) ssd_scan_kernel<4, 16, 16><<<grid, 256, 0, s_>>>(p); else ssd_scan_kernel<4, 16, 8><<<grid, 256, 0, s_>>>(p); }
+        else if (n_state <= 128) { if (longer) ssd_scan_kernel<8, 16, 16><<<grid, 256, 0, s_>>>(p); else ssd_scan_kernel<8, 16, 8><<<grid, 256, 0, s_>>>(p); }
         else ssd_scan_kernel<16, 16, 8><<<grid, 256, 0, s_>>>(p);
     }
     LAUNCH_OK(); return 0;

@@ -208,7 +208,7 @@ def test_attention_with_distance_bias_and_keys_that_stand_out(lib, dtype, Hh, G,
     scale = 1.0 / math.sqrt(d)
     u = rng.standard_normal(d); u /= np.linalg.norm(u)
     first = L - n_new
-    pairs = [(L - 1, max(0, L - 1 - 257)), (L - 1, 0)]
+    pairs = [(L - 1, max(0, L - 1 - 257)), (L - 1, 0), (L - 1, ((L - 1) // bs) * bs), (L - 1, ((L - 1) // bs) * bs - 1)]
     if n_new > 4:
         pairs += [(first + 1, (first // bs) * bs), (first + 2, max(0, (first // bs) * bs - 1)), (first + 3, first + 3), (first, max(0, first - 129))]
     for i, j in pairs:                                                    # score of (i, j) = 30 before the bias: far above the rest
