@@ -378,7 +378,7 @@ int mi355_hyb_ssd_scan(float* y, float* state, int64_t state_stride, const float
                        const uint32_t* cu_seqlens_q, const int32_t* state_slots, int32_t num_seqs, int32_t num_tokens, int32_t heads,
                        int32_t groups, int32_t n_state, int32_t vdim, int64_t stream) {
     if (!y || !state || !xbc || !dt_in || !a_log || !dt_bias || !context_lens || !cu_seqlens_q || !state_slots) return -1;
-    if (heads <= 0 || groups <= 0 || heads % groups || n_state <= 0 || n_state > 256 || vdim <= 0) return -1;
+    if (heads <= 0 || groups <= 0 || heads % groups || n_state <= 0 || n_state > 512 || vdim <= 0) return -1;
     if (ldx < heads * vdim + 2 * groups * n_state || ldd < heads) return -1;
     if (num_seqs <= 0 || num_tokens <= 0) return 0;
     SsdArgs p{y, state, state_stride, xbc, ldx, dt_in, ldd, a_log, dt_bias, skip, context_lens, cu_seqlens_q, state_slots, heads, groups, n_state, vdim};
@@ -394,7 +394,8 @@ int mi355_hyb_ssd_scan(float* y, float* state, int64_t state_stride, const float
         const bool longer = num_tokens > 8 * num_seqs;
         if (n_state <= 64) { if (longer) ssd_scan_kernel<4, 16, 16><<<grid, 256, 0, s_>>>(p); else ssd_scan_kernel<4, 16, 8><<<grid, 256, 0, s_>>>(p); }
         else if (n_state <= 128) { if (longer) ssd_scan_kernel<8, 16, 16><<<grid, 256, 0, s_>>>(p); else ssd_scan_kernel<8, 16, 8><<<grid, 256, 0, s_>>>(p); }
-        else ssd_scan_kernel<16, 16, 8><<<grid, 256, 0, s_>>>(p);
+        else if (n_state <= 256) ssd_scan_kernel<16, 16, 8><<<grid, 256, 0, s_>>>(p);
+        else ssd_scan_kernel<32, 16, 4><<<grid, 256, 0, s_>>>(p);       // (stages of 4 tokens: two stages of B and C rows of 512 states fill LDS)
     }
     LAUNCH_OK(); return 0;
 }

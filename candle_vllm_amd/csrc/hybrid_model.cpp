@@ -151,7 +151,7 @@ bool layer_ok(const mi355_hybrid_layer& c) {
     const bool delta = c.mixer == MI355_HYB_MIX_PARALLEL || c.mixer == MI355_HYB_MIX_DELTA;
     if (c.mixer < 0 || c.mixer > MI355_HYB_MIX_SSD || c.share_with < 0) return false;
     if (c.mixer == MI355_HYB_MIX_SSD) {
-        if (c.d_heads <= 0 || c.d_kv_heads <= 0 || c.d_heads % c.d_kv_heads || c.d_dim <= 0 || c.d_dim > 256 || c.d_vdim <= 0) return false;
+        if (c.d_heads <= 0 || c.d_kv_heads <= 0 || c.d_heads % c.d_kv_heads || c.d_dim <= 0 || c.d_dim > 512 || c.d_vdim <= 0) return false;
         if (c.d_conv < 1 || c.d_conv > 16 || c.d_norm_groups < 1 || (c.d_heads * c.d_vdim) % c.d_norm_groups) return false;
     }
     if (c.a_q_rank < 0 || c.kv_from < 0 || c.side_dim < 0 || c.side_col < 0 || c.depth_terms < 0 || c.moe_groups < 0) return false;

@@ -404,7 +404,7 @@ int mi355_hyb_gate_group_norm(void* out, int32_t out_dtype, const float* y, cons
 /* state-space scan over the new tokens of every sequence, state f32 [slots] x [heads, n_state, vdim] (stride in floats).
  * xbc f32 [T, ldx]: x (heads x vdim) at 0, B (groups x n_state) behind it, C behind that, all behind the convolution and silu;
  * dt_in f32 rows of ldd: the raw step per head; dt = softplus(dt_in + dt_bias[h]), decay = exp(-exp(a_log[h]) dt);
- * S <- decay S + dt B x^T;  y f32 [T, heads, vdim] = S^T C + skip[h] x.  Head h reads group h / (heads / groups). */
+ * S <- decay S + dt B x^T;  y f32 [T, heads, vdim] = S^T C + skip[h] x.  Head h reads group h / (heads / groups).  n_state <= 512. */
 int mi355_hyb_ssd_scan(float* y, float* state, int64_t state_stride, const float* xbc, int32_t ldx, const float* dt_in, int32_t ldd,
                        const float* a_log, const float* dt_bias, const float* skip, const uint32_t* context_lens,
                        const uint32_t* cu_seqlens_q, const int32_t* state_slots, int32_t num_seqs, int32_t num_tokens, int32_t heads,

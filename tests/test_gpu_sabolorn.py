@@ -104,7 +104,8 @@ def test_layer_norm_and_rms_norm_of_rows(lib, dtype, T, W, ld):
     assert np.abs(host_dt(out, dtype) - want).max() < tol(dtype, 5e-5) * max(1.0, np.abs(want).max())
 
 
-@pytest.mark.parametrize("heads,G,N,vd", [(4, 2, 24, 16), (3, 1, 5, 1), (2, 2, 64, 24), (6, 3, 128, 64), (1, 1, 200, 80), (5, 5, 16, 70), (2, 1, 33, 8)])
+@pytest.mark.parametrize("heads,G,N,vd", [(4, 2, 24, 16), (3, 1, 5, 1), (2, 2, 64, 24), (6, 3, 128, 64), (1, 1, 200, 80), (5, 5, 16, 70), (2, 1, 33, 8), (2, 2, 400, 20),
+                                          (1, 1, 512, 3)])
 def test_state_space_scan_over_portions_and_reused_slots(lib, heads, G, N, vd):
     """two sequences of unequal length side by side, in portions of 1, 2, 9, ... tokens that continue from their slots; the slots
     hold stale values at the start (position 0 starts from zero); then a new sequence takes over a used slot"""
