@@ -3,7 +3,9 @@
 // attention behind a short convolution with mixed head weights) and an optional feed-forward; x <- x + norm(mixer(x)),
 // x <- x + norm(ff(x)) -- or, with residual_form 1, x <- norm(alpha x + mixer(x)), x <- norm(alpha x + ff(x)) -- the sublayers read
 // x itself; residual_form 2 puts a norm on both sides, x <- x + norm(sub(pre_norm(x))), optionally with a short causal convolution
-// added to the mixer's input.  The feed-forward is a dense gate/up form or a mixture of experts (router, grouped expert products over
+// added to the mixer's input; residual_form 3 has ONE norm per layer that mixer and feed-forward both read, x <- x + mixer(h) + ff(h),
+// then the token's side input and the average over the depth (a state-space mixer and an ungated feed-forward belong to that form's
+// design).  The feed-forward is a dense gate/up form or a mixture of experts (router, grouped expert products over
 // device-built blocks, shared expert).  A layer may run on another layer's weights (share_with) and still owns its pages and state.  Like the llama-family host layers
 // (host_model.cpp, dense_model.cpp) it owns the weights, the K/V pages and the activation buffers and enqueues one step on a
 // stream; unlike them it owns a pool of recurrent state (one slot per live sequence, handed out by the block engine) and runs

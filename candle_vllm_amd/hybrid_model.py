@@ -1,7 +1,7 @@
 """Python harness over the `mi355_hybrid_*` handle (include/mi355_hybrid.h): layer-list models whose layers mix tokens by
 sliding-window attention with a sink, a gated delta rule, a minGRU, attention and delta rule side by side, latent attention, or
-attention behind a short convolution with mixed head weights, with dense or mixture-of-experts feed-forwards.  The Sogodra, Vivazen
-and Kerolorn designs are read here: a design's
+attention behind a short convolution with mixed head weights, or a state-space mixer, with dense or mixture-of-experts
+feed-forwards.  The Sogodra, Vivazen, Kerolorn and Sabolorn designs are read here: a design's
 config.json (`architecture`, `layers`, `norm`, `vocab`, `width`, ...) becomes the C structs, its tensors are concatenated into the
 host layer's slots.  No CPU fallback; torch only holds device buffers."""
 import ctypes

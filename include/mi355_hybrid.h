@@ -2,7 +2,8 @@
  * layer has -- sliding-window attention with a softmax sink, a gated delta rule (recurrent matrix state), a minGRU (recurrent vector
  * state), attention and delta rule side by side, latent attention (keys and values read off one cached latent vector per token), or
  * attention behind a short convolution whose heads' softmax weights are mixed -- and which feed-forward (dense gate/up forms or a
- * mixture of experts).  The Sogodra, Vivazen and Kerolorn designs are its users.
+ * mixture of experts), or a state-space mixer with a scalar decay per head.  The Sogodra, Vivazen, Kerolorn and Sabolorn designs are
+ * its users.
  *
  * What differs from the llama-family host layers (mi355_llama_*, mi355_dense_*):
  *   - the residual stream, norms, attention scores, decays, gates of a recurrence and the recurrent state are f32 in both dtypes;
